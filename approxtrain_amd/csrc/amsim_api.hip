@@ -1,0 +1,331 @@
+// extern "C" entry points: each one describes its reduction to the GEMM engine
+// (which operand runs over the lanes, which is wave-uniform, how the lane
+// operand is gathered) and launches it.  No device memory is allocated here.
+#include "amsim_internal.h"
+
+#include <algorithm>
+
+namespace amsim {
+void set_split_k(int mode);
+}
+
+using namespace amsim;
+
+namespace {
+
+inline int tn_for(int64_t J) { return J >= 9 ? 16 : J >= 5 ? 8 : J >= 3 ? 4 : (int)std::max<int64_t>(J, 1); }
+
+inline int64_t padded_work(int64_t R, int64_t J)
+{
+    const int tn = tn_for(J);
+    return ((R + 63) / 64 * 64) * ((J + tn - 1) / tn * tn);
+}
+
+// true: rows of C over the lanes (lane operand = op(A)); false: columns of C
+// over the lanes (lane operand = op(B)).  Picks the orientation that wastes
+// fewer lanes / accumulators on padding.
+inline bool lanes_along_m(int64_t M, int64_t N) { return padded_work(M, N) <= padded_work(N, M); }
+
+struct GemmCall {
+    int transA, transB, swap;
+    int64_t M, N, K;
+    const float *A; int64_t lda;
+    const float *B; int64_t ldb;
+    float *C; int64_t ldc;
+    int64_t batch, strideA, strideB, strideC;
+};
+
+GemmDesc describe(const GemmCall &g)
+{
+    GemmDesc d;
+    d.K = g.K;
+    d.batch = (int)g.batch;
+    d.out = g.C;
+    d.out_batch_stride = g.strideC;
+    if (lanes_along_m(g.M, g.N)) {
+        d.R = g.M; d.J = g.N;
+        d.p.kind = P_DENSE; d.p.base = g.A; d.p.batch_stride = g.strideA;
+        d.p.sr = g.transA ? 1 : g.lda; d.p.sk = g.transA ? g.lda : 1;
+        d.q.kind = Q_DENSE; d.q.base = g.B; d.q.batch_stride = g.strideB;
+        d.q.batches = (g.batch > 1 && g.strideB != 0) ? (int)g.batch : 1;
+        d.q.sk = g.transB ? 1 : g.ldb; d.q.sj = g.transB ? g.ldb : 1;
+        d.so_r = g.ldc; d.so_j = 1;
+        d.lane_first = !g.swap;
+    } else {
+        d.R = g.N; d.J = g.M;
+        d.p.kind = P_DENSE; d.p.base = g.B; d.p.batch_stride = g.strideB;
+        d.p.sr = g.transB ? g.ldb : 1; d.p.sk = g.transB ? 1 : g.ldb;
+        d.q.kind = Q_DENSE; d.q.base = g.A; d.q.batch_stride = g.strideA;
+        d.q.batches = (g.batch > 1 && g.strideA != 0) ? (int)g.batch : 1;
+        d.q.sk = g.transA ? g.lda : 1; d.q.sj = g.transA ? 1 : g.lda;
+        d.so_r = 1; d.so_j = g.ldc;
+        d.lane_first = g.swap != 0;
+    }
+    return d;
+}
+
+int gemm_call(amsim_lut_t lut, const GemmCall &g, void *ws, size_t ws_bytes, void *stream)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (g.M < 0 || g.N < 0 || g.K < 0 || g.batch < 0) return fail(AMSIM_ERR_INVALID, "negative extent");
+    if (g.M == 0 || g.N == 0 || g.batch == 0) return AMSIM_OK;
+    if (g.C == nullptr || (g.K > 0 && (g.A == nullptr || g.B == nullptr)))
+        return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    const int64_t min_lda = g.transA ? g.M : g.K, min_ldb = g.transB ? g.K : g.N;
+    if (g.lda < min_lda || g.ldb < min_ldb || g.ldc < g.N)
+        return fail(AMSIM_ERR_INVALID, "leading dimension smaller than the row length");
+    return run_gemm(lut->l, describe(g), ws, ws_bytes, static_cast<hipStream_t>(stream));
+}
+
+size_t gemm_ws(const GemmCall &g)
+{
+    if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) return 0;
+    GemmDesc d = describe(g);
+    return gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
+}
+
+bool fits_int32(int64_t elements) { return elements < (1ll << 31); }
+
+}  // namespace
+
+extern "C" {
+
+int amsim_set_split_k(int mode)
+{
+    amsim::set_split_k(mode);
+    return AMSIM_OK;
+}
+
+int amsim_mul_f32(amsim_lut_t lut, const float *a, const float *b, float *out, size_t n, void *stream)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (n && (!a || !b || !out)) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    return launch_mul(lut->l, a, b, out, n, static_cast<hipStream_t>(stream));
+}
+
+size_t amsim_gemm_workspace_bytes(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch)
+{
+    // sized for per-item operands (no broadcast), the larger case
+    GemmCall g{transA, transB, 0, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, batch, 1, 1, 1};
+    return gemm_ws(g);
+}
+
+int amsim_gemm_f32(amsim_lut_t lut, int transA, int transB, int swap_operands, int64_t M, int64_t N, int64_t K,
+                   const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc,
+                   int64_t batch, int64_t strideA, int64_t strideB, int64_t strideC, void *workspace,
+                   size_t workspace_bytes, void *stream)
+{
+    GemmCall g{transA, transB, swap_operands, M, N, K, A, lda, B, ldb, C, ldc, batch, strideA, strideB, strideC};
+    return gemm_call(lut, g, workspace, workspace_bytes, stream);
+}
+
+// ---- convolution ------------------------------------------------------------------
+
+size_t amsim_convam_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth, int filter_rows,
+                                    int filter_cols, int in_depth)
+{
+    return gemm_workspace_bytes((int64_t)batch * out_rows * out_cols, out_depth,
+                                (int64_t)filter_rows * filter_cols * in_depth, 1, 1);
+}
+
+int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
+                     int out_cols, int out_depth, int stride_cols, int stride_rows, int filter_left_offset,
+                     int filter_top_offset, int filter_rows, int filter_cols, int in_depth, int input_cols,
+                     int input_rows, const float *filter, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (batch < 0 || out_rows < 0 || out_cols < 0 || out_depth < 0 || filter_rows < 0 || filter_cols < 0 ||
+        in_depth < 0 || input_cols < 0 || input_rows < 0 || stride_cols < 1 || stride_rows < 1)
+        return fail(AMSIM_ERR_INVALID, "bad convolution geometry");
+    const int64_t R = (int64_t)batch * out_rows * out_cols;
+    if (R == 0 || out_depth == 0) return AMSIM_OK;
+    if (!input_data || !output_data || !filter) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    if (!fits_int32((int64_t)batch * input_rows * input_cols * in_depth))
+        return fail(AMSIM_ERR_UNSUPPORTED, "input tensor has 2^31 or more elements");
+    // im2col rows (b, oy, ox) x columns (fy, fx, c)  [cuda_kernel.cu:35-60], filter as the [K][OC] matrix
+    GemmDesc d;
+    d.R = R; d.J = out_depth; d.K = (int64_t)filter_rows * filter_cols * in_depth;
+    d.p.kind = P_PATCH; d.p.base = input_data;
+    d.p.B = batch; d.p.GH = out_rows; d.p.GW = out_cols;
+    d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = in_depth;
+    d.p.sy = stride_rows; d.p.sx = stride_cols; d.p.pt = filter_top_offset; d.p.pl = filter_left_offset;
+    d.p.dy = 1; d.p.dx = 1; d.p.VH = input_rows; d.p.VW = input_cols; d.p.SH = input_rows; d.p.SW = input_cols;
+    d.q.kind = Q_DENSE; d.q.base = filter; d.q.sk = out_depth; d.q.sj = 1;
+    d.out = output_data; d.so_r = out_depth; d.so_j = 1;
+    d.lane_first = true;  // P(input, filter)
+    return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+size_t amsim_convam_input_grad_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
+                                               int filter_rows, int filter_cols, int out_depth)
+{
+    return gemm_workspace_bytes((int64_t)batch * input_rows * input_cols, in_depth,
+                                (int64_t)filter_rows * filter_cols * out_depth, 1, 1);
+}
+
+int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_grad_width, int hole_grad_height,
+                                int pad_top, int pad_left, const float *filter, int filter_rows, int filter_cols,
+                                int out_depth, int stride_rows, int stride_cols, int batch, int input_rows,
+                                int input_cols, int in_depth, float *output, int out_rows, int out_cols,
+                                void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (batch < 0 || input_rows < 0 || input_cols < 0 || in_depth < 0 || filter_rows < 0 || filter_cols < 0 ||
+        out_depth < 0 || out_rows < 0 || out_cols < 0 || stride_cols < 1 || stride_rows < 1)
+        return fail(AMSIM_ERR_INVALID, "bad convolution geometry");
+    if (out_rows > 0 && out_cols > 0 &&
+        (hole_grad_height != (out_rows - 1) * stride_rows + 1 || hole_grad_width != (out_cols - 1) * stride_cols + 1))
+        return fail(AMSIM_ERR_INVALID, "hole_grad extent must be (out - 1) * stride + 1");
+    const int64_t R = (int64_t)batch * input_rows * input_cols;
+    if (R == 0 || in_depth == 0) return AMSIM_OK;
+    if (!grad || !output || !filter) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    if (!fits_int32((int64_t)batch * out_rows * out_cols * out_depth))
+        return fail(AMSIM_ERR_UNSUPPORTED, "gradient tensor has 2^31 or more elements");
+    // rows (b, y, x) of the input x columns (fy, fx, oc) of the zero-dilated,
+    // back-padded gradient [cuda_kernel.cu:463-502]; the flipped, I/O-swapped
+    // filter [reverseNswapdim23.cu:16] is produced by the operand pre-pass.
+    GemmDesc d;
+    d.R = R; d.J = in_depth; d.K = (int64_t)filter_rows * filter_cols * out_depth;
+    d.p.kind = P_PATCH; d.p.base = grad;
+    d.p.B = batch; d.p.GH = input_rows; d.p.GW = input_cols;
+    d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = out_depth;
+    d.p.sy = 1; d.p.sx = 1; d.p.pt = pad_top; d.p.pl = pad_left;
+    d.p.dy = stride_rows; d.p.dx = stride_cols; d.p.VH = hole_grad_height; d.p.VW = hole_grad_width;
+    d.p.SH = out_rows; d.p.SW = out_cols;
+    d.q.kind = Q_FLIP; d.q.base = filter; d.q.KH = filter_rows; d.q.KW = filter_cols; d.q.IC = in_depth;
+    d.q.OC = out_depth;
+    d.out = output; d.so_r = in_depth; d.so_j = 1;
+    d.lane_first = true;  // P(grad, filter)
+    return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth,
+                                                int filter_rows, int filter_cols, int in_depth)
+{
+    return gemm_workspace_bytes((int64_t)filter_rows * filter_cols * in_depth, out_depth,
+                                (int64_t)batch * out_rows * out_cols, 1, 1);
+}
+
+int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const float *grad, int input_rows,
+                                 int input_cols, int batch, int in_depth, int out_cols, int out_rows,
+                                 int out_depth, int filter_left_offset, int filter_top_offset, int stride_rows,
+                                 int stride_cols, int filter_cols, int filter_rows, float *output, void *workspace,
+                                 size_t workspace_bytes, void *stream)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (batch < 0 || input_rows < 0 || input_cols < 0 || in_depth < 0 || filter_rows < 0 || filter_cols < 0 ||
+        out_depth < 0 || out_rows < 0 || out_cols < 0 || stride_cols < 1 || stride_rows < 1)
+        return fail(AMSIM_ERR_INVALID, "bad convolution geometry");
+    const int64_t R = (int64_t)filter_rows * filter_cols * in_depth;
+    if (R == 0 || out_depth == 0) return AMSIM_OK;
+    if (!output) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    const int64_t K = (int64_t)batch * out_rows * out_cols;
+    if (K > 0 && (!input || !grad)) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    if (!fits_int32((int64_t)batch * input_rows * input_cols * in_depth))
+        return fail(AMSIM_ERR_UNSUPPORTED, "input tensor has 2^31 or more elements");
+    // rows (fy, fx, c) of the filter x reduction over (b, oy, ox)
+    // [cuda_kernel.cu:327-353, 417-425]; the gradient is the [K][OC] matrix
+    GemmDesc d;
+    d.R = R; d.J = out_depth; d.K = K;
+    d.p.kind = P_GF; d.p.base = input;
+    d.p.B = batch; d.p.GH = out_rows; d.p.GW = out_cols;
+    d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = in_depth;
+    d.p.sy = stride_rows; d.p.sx = stride_cols; d.p.pt = filter_top_offset; d.p.pl = filter_left_offset;
+    d.p.SH = input_rows; d.p.SW = input_cols; d.p.VH = input_rows; d.p.VW = input_cols;
+    d.q.kind = Q_DENSE; d.q.base = grad; d.q.sk = out_depth; d.q.sj = 1;
+    d.out = output; d.so_r = out_depth; d.so_j = 1;
+    d.lane_first = true;  // P(input, grad)
+    return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+// ---- dense ----------------------------------------------------------------------------
+
+size_t amsim_denseam_workspace_bytes(int batch, int units, int input_width)
+{
+    // the largest of the three GEMMs of the layer
+    GemmCall f{0, 0, 0, batch, units, input_width, nullptr, 0, nullptr, 0, nullptr, 0, 1, 0, 0, 0};
+    GemmCall w{1, 0, 0, input_width, units, batch, nullptr, 0, nullptr, 0, nullptr, 0, 1, 0, 0, 0};
+    GemmCall x{0, 1, 1, batch, input_width, units, nullptr, 0, nullptr, 0, nullptr, 0, 1, 0, 0, 0};
+    return std::max(gemm_ws(f), std::max(gemm_ws(w), gemm_ws(x)));
+}
+
+int amsim_denseam_f32(amsim_lut_t lut, const float *inputs, const float *weights, float *output, int batch,
+                      int units, int input_width, void *workspace, size_t workspace_bytes, void *stream)
+{
+    // denseam_kernel.cu:38-41: P(input, weight)
+    GemmCall g{0, 0, 0, batch, units, input_width, inputs, input_width, weights, units, output, units, 1, 0, 0, 0};
+    return gemm_call(lut, g, workspace, workspace_bytes, stream);
+}
+
+int amsim_denseam_weight_grad_f32(amsim_lut_t lut, const float *input, const float *grads, float *output,
+                                  int batch, int units, int input_width, void *workspace, size_t workspace_bytes,
+                                  void *stream)
+{
+    // denseam_kernel.cu:64-67: dW[k][j] = sum_i P(input[i][k], grads[i][j])
+    GemmCall g{1, 0, 0, input_width, units, batch, input, input_width, grads, units, output, units, 1, 0, 0, 0};
+    return gemm_call(lut, g, workspace, workspace_bytes, stream);
+}
+
+int amsim_denseam_input_grad_f32(amsim_lut_t lut, const float *weight, const float *grads, float *output,
+                                 int batch, int units, int input_width, void *workspace, size_t workspace_bytes,
+                                 void *stream)
+{
+    // denseam_kernel.cu:91-94: dX[i][k] = sum_j P(weight[k][j], grads[i][j]) -- weight is the first LUT operand
+    GemmCall g{0, 1, 1, batch, input_width, units, grads, units, weight, units, output, input_width, 1, 0, 0, 0};
+    return gemm_call(lut, g, workspace, workspace_bytes, stream);
+}
+
+// ---- matmul ---------------------------------------------------------------------------
+
+static int matmul_call(int batch_a, int batch_b, int row_a, int col_a, int row_b, int col_b, GemmCall *g)
+{
+    if (batch_a < 0 || batch_b < 0 || row_a < 0 || col_a < 0 || row_b < 0 || col_b < 0)
+        return fail(AMSIM_ERR_INVALID, "negative extent");
+    if (col_a != row_b) return fail(AMSIM_ERR_INVALID, "Does not meet cols of mat a is equal rows of mat b");
+    if (batch_a > 1 && batch_b > 1 && batch_a != batch_b)
+        return fail(AMSIM_ERR_INVALID, "Does not meet batch of mat a is equal batch of matb");
+    const int nb = std::max(std::max(batch_a, batch_b), 1);
+    *g = GemmCall{0, 0, 0, row_a, col_b, col_a, nullptr, col_a, nullptr, col_b, nullptr, col_b, nb,
+                  batch_a > 1 ? (int64_t)row_a * col_a : 0, batch_b > 1 ? (int64_t)row_b * col_b : 0,
+                  (int64_t)row_a * col_b};
+    return AMSIM_OK;
+}
+
+size_t amsim_matmulam_workspace_bytes(int batch_a, int batch_b, int row_a, int col_a, int row_b, int col_b)
+{
+    GemmCall g;
+    if (matmul_call(batch_a, batch_b, row_a, col_a, row_b, col_b, &g) != AMSIM_OK) return 0;
+    return gemm_ws(g);
+}
+
+int amsim_matmulam_f32(amsim_lut_t lut, const float *a, const float *b, int batch_a, int batch_b, int row_a,
+                       int col_a, int row_b, int col_b, float *out, void *workspace, size_t workspace_bytes,
+                       void *stream)
+{
+    GemmCall g;
+    int rc = matmul_call(batch_a, batch_b, row_a, col_a, row_b, col_b, &g);
+    if (rc != AMSIM_OK) return rc;
+    g.A = a; g.B = b; g.C = out;
+    return gemm_call(lut, g, workspace, workspace_bytes, stream);
+}
+
+// ---- geometry -------------------------------------------------------------------------
+
+int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, int *out_size, int *pad_before)
+{
+    if (in_size < 0 || filter_size < 1 || stride < 1 || !out_size || !pad_before)
+        return fail(AMSIM_ERR_INVALID, "bad window geometry");
+    if (padding == AMSIM_PADDING_VALID) {
+        *out_size = in_size - filter_size + stride >= 0 ? (in_size - filter_size + stride) / stride : 0;
+        *pad_before = 0;
+    } else if (padding == AMSIM_PADDING_SAME) {
+        *out_size = (in_size + stride - 1) / stride;
+        const int total = std::max((*out_size - 1) * stride + filter_size - in_size, 0);
+        *pad_before = total / 2;
+    } else {
+        return fail(AMSIM_ERR_INVALID, "padding must be AMSIM_PADDING_VALID or AMSIM_PADDING_SAME");
+    }
+    return AMSIM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,49 @@
+// Device-side building blocks of the approximate product (gfx950).
+#ifndef AMSIM_DEVICE_H_
+#define AMSIM_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace amsim {
+
+__device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
+
+// An operand is "safe" when it is a zero or a normal number with biased
+// exponent in [64, 190].  For two safe operands the product of the functional
+// models (lut/FPmultMBM_fast16.inl:45-134) reduces to
+//     sign(a)^sign(b) | (ea + eb - 127 + carry) << 23 | mantissa
+// with no underflow, overflow or special case: ea + eb lies in [128, 380], and
+// a zero operand gives a zero product.  Everything else takes am_exact().
+__device__ __forceinline__ bool operand_unsafe(uint32_t bits)
+{
+    uint32_t mag = bits & 0x7fffffffu;
+    uint32_t e = mag >> 23;
+    return mag != 0u && (e - 64u) > 126u;
+}
+
+// Full-domain product.  `entry16` is the LUT byte (carry << 7 | mantissa
+// left-aligned in 7 bits) shifted left by 16, i.e. carry << 23 | mantissa.
+// Restates the exponent / special-case logic of the C functional models:
+//   p = a * b (IEEE, subnormals kept) supplies sign, exponent and class;
+//   exp(p) == 255 -> p itself (inf / NaN pass through, :99-101);
+//   exp(p) == 0   -> +0 (:102-104);
+//   else exponent = exp(p) - accurate_normalised + carry (:106-112), where
+//   accurate_normalised is whether the exact significand product, rounded to
+//   nearest even, reached 2.0 (:58-96).
+__device__ __forceinline__ float am_exact(uint32_t at, uint32_t bt, uint32_t entry16)
+{
+    float p = u2f(at) * u2f(bt);
+    uint32_t pt = f2u(p);
+    uint32_t pe = (pt >> 23) & 255u;
+    if (pe == 255u) return p;
+    if (pe == 0u) return 0.0f;
+    float sa = u2f(0x3f800000u | (at & 0x7fffffu));
+    float sb = u2f(0x3f800000u | (bt & 0x7fffffu));
+    uint32_t acc = (sa * sb >= 2.0f) ? 1u : 0u;
+    return u2f((pt & 0x80000000u) + ((pe - acc) << 23) + entry16);
+}
+
+}  // namespace amsim
+#endif

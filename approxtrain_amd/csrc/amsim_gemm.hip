@@ -1,0 +1,513 @@
+// LUT-multiply GEMM engine for gfx950 (MI355X).
+//
+// out(r, j) = sum_k P(p(r, k), q(k, j)),  P = approximate product through a
+// mantissa LUT, FP32 accumulation in ascending k.
+//
+// Mapping to the machine (VALU/LDS-bound by construction; no MFMA because the
+// product is not an IEEE multiply):
+//   * r runs over the 64 lanes of a wavefront, j is wave-uniform.  At every
+//     LUT gather all lanes share the uniform operand's mantissa, so the 64
+//     addresses fall into ONE 2^m-byte row of the byte-wide LUT image in LDS:
+//     at most 32 distinct dwords, one per bank -> no bank conflicts ever.
+//   * the uniform operand q is pre-decoded once per call into
+//     (sign|exponent as a power-of-two float, LUT row offset) pairs and read
+//     through the scalar cache (s_load), so it costs no VALU and no LDS.
+//   * the lane operand p is staged through LDS in [k][r] order by coalesced
+//     loads (dense, im2col-style patches, or filter-gradient gathers computed
+//     on the fly: no im2col / flipped-filter temporaries in HBM).
+//   * per MAC: v_add (LUT address), ds_read_u8, v_mul (2^ea * 2^eb),
+//     v_lshl_add (byte -> 1.mant * 2^carry as a float), v_fma (accumulate).
+//     t * f is exact (power of two times an 8-bit significand), so the fused
+//     multiply-add rounds exactly like the reference's product-then-add.
+//   * operands outside the "safe" range (subnormal, inf, NaN, |x| < 2^-63 or
+//     >= 2^64) flag their 32-deep k chunk; flagged chunks take the exact
+//     full-domain product instead (wave-uniform branch), so results are
+//     bit-exact everywhere without taxing the fast path.
+#include "amsim_internal.h"
+#include "amsim_device.h"
+
+#include <algorithm>
+#include <atomic>
+
+namespace amsim {
+
+constexpr int KC = 32;        // reduction depth of one staged chunk
+constexpr int WG_THREADS = 256;
+constexpr int LUT_LDS_BYTES = 16384;
+constexpr int TARGET_WAVES = 4096;
+
+static std::atomic<int> g_split_k{1};
+
+typedef const __attribute__((address_space(4))) uint2 *cq2_t;
+typedef const __attribute__((address_space(4))) uint32_t *cq1_t;
+
+struct KArgs {
+    PDesc p;
+    const uint8_t *lut_img;  // byte image: (uniform mantissa << m) | lane mantissa
+    int lut_bytes;
+    int m;
+    int lane_first;
+    const uint2 *qd;         // [qb][Kp][Jp] (t bits, row offset)
+    const uint32_t *qraw;    // [qb][Kp][Jp] raw bits
+    const uint32_t *qflags;  // [qb][nchunks]
+    int q_batches;
+    int64_t R, J, K;
+    int Jp, nchunks, nsplit, chunks_per_split;
+    float *out;
+    int64_t so_r, so_j, out_batch_stride;
+    float *partial;          // [nsplit][batch][Rp][Jp] when nsplit > 1
+    int64_t Rp;
+    int batch;
+};
+
+// ---------------------------------------------------------------------------
+// uniform-operand pre-pass
+// ---------------------------------------------------------------------------
+struct QArgs {
+    QDesc q;
+    int64_t K, J;
+    int Jp, nchunks, m;
+    uint2 *qd;
+    uint32_t *qraw;
+    uint32_t *qflags;
+};
+
+__global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
+{
+    const int ch = blockIdx.x, qb = blockIdx.y;
+    const float *base = a.q.base + (int64_t)qb * a.q.batch_stride;
+    const size_t plane = (size_t)a.nchunks * KC * a.Jp;
+    uint2 *qd = a.qd + (size_t)qb * plane + (size_t)ch * KC * a.Jp;
+    uint32_t *qraw = a.qraw + (size_t)qb * plane + (size_t)ch * KC * a.Jp;
+    int unsafe = 0;
+    const int n = KC * a.Jp;
+    for (int e = threadIdx.x; e < n; e += WG_THREADS) {
+        const int kk = e / a.Jp, j = e - kk * a.Jp;
+        const int64_t k = (int64_t)ch * KC + kk;
+        uint32_t raw = 0;
+        if (k < a.K && j < a.J) {
+            if (a.q.kind == Q_DENSE) {
+                raw = f2u(base[k * a.q.sk + j * a.q.sj]);
+            } else {
+                const int oc = (int)(k % a.q.OC);
+                const int t = (int)(k / a.q.OC);
+                const int fx = t % a.q.KW, fy = t / a.q.KW;
+                raw = f2u(base[(((int64_t)(a.q.KH - 1 - fy) * a.q.KW + (a.q.KW - 1 - fx)) * a.q.IC + j) * a.q.OC + oc]);
+            }
+        }
+        unsafe |= operand_unsafe(raw) ? 1 : 0;
+        const uint32_t mant = (raw & 0x7fffffu) >> (23 - a.m);
+        qd[e] = make_uint2(raw & 0xff800000u, mant << a.m);
+        qraw[e] = raw;
+    }
+    unsafe = __syncthreads_or(unsafe);
+    if (threadIdx.x == 0) a.qflags[(size_t)qb * a.nchunks + ch] = (uint32_t)unsafe;
+}
+
+// ---------------------------------------------------------------------------
+// lane-operand loaders
+// ---------------------------------------------------------------------------
+// Row bookkeeping kept in LDS: three ints per local row.
+//   P_PATCH: {source offset of image b, y*sy - pt, x*sx - pl}; invalid rows get
+//            a y origin far outside the source.
+//   P_GF:    {(fy*SW + fx)*C + c, fy, fx}; invalid rows get fy far outside.
+__device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t row0, int rows, int *ri)
+{
+    for (int rl = threadIdx.x; rl < rows; rl += WG_THREADS) {
+        const int64_t r = row0 + rl;
+        int a0 = 0, a1 = -(1 << 28), a2 = 0;
+        if (r < R) {
+            if (p.kind == P_PATCH) {
+                const int x = (int)(r % p.GW);
+                const int64_t t = r / p.GW;
+                const int y = (int)(t % p.GH);
+                const int b = (int)(t / p.GH);
+                a0 = b * p.SH * p.SW * p.C;
+                a1 = y * p.sy - p.pt;
+                a2 = x * p.sx - p.pl;
+            } else if (p.kind == P_GF) {
+                const int c = (int)(r % p.C);
+                const int t = (int)(r / p.C);
+                const int fx = t % p.KW, fy = t / p.KW;
+                a0 = (fy * p.SW + fx) * p.C + c;
+                a1 = fy;
+                a2 = fx;
+            }
+        }
+        ri[rl * 3 + 0] = a0;
+        ri[rl * 3 + 1] = a1;
+        ri[rl * 3 + 2] = a2;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// main kernel
+// ---------------------------------------------------------------------------
+// TN       outputs per lane (uniform-dimension tile of one wave)
+// WR       row tiles per workgroup (waves are arranged WR x 4/WR)
+// PK       lane-operand loader
+// ALONG_K  staging threads run along k (source contiguous in k) or along r
+template <int TN, int WR, int PK, bool ALONG_K>
+__global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
+{
+    constexpr int WC = 4 / WR;
+    constexpr int ROWS = 64 * WR;
+    constexpr int RS = ROWS + (ALONG_K ? 1 : 0);  // padded row stride: conflict-free transposing stores
+    constexpr int ELEMS = ROWS * KC / WG_THREADS;
+
+    __shared__ __align__(16) uint8_t lut_s[LUT_LDS_BYTES];
+    __shared__ uint32_t Pt[KC * RS];
+    __shared__ int rowinfo[ROWS * 3];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave / WC, wc = wave % WC;
+    const int bz = blockIdx.z / a.nsplit, split = blockIdx.z % a.nsplit;
+    const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+    const int j0 = (blockIdx.y * WC + wc) * TN;
+    const bool active = j0 < a.J;
+    const int m = a.m;
+
+    for (int i = tid * 16; i < a.lut_bytes; i += WG_THREADS * 16)
+        *reinterpret_cast<uint4 *>(lut_s + i) = *reinterpret_cast<const uint4 *>(a.lut_img + i);
+    if (PK != P_DENSE) fill_rowinfo(a.p, a.R, row0, ROWS, rowinfo);
+    __syncthreads();
+
+    const float *pbase = a.p.base + (int64_t)bz * a.p.batch_stride;
+    const int qb = a.q_batches > 1 ? bz : 0;
+    const size_t qplane = (size_t)a.nchunks * KC * a.Jp;
+    // The pre-decoded uniform operand was written by an earlier kernel and is
+    // read-only here: address it through the constant address space so that the
+    // wave-uniform reads become scalar loads (s_load) into SGPRs.
+    const cq2_t qd = (cq2_t)(uintptr_t)(a.qd + (size_t)qb * qplane);
+    const cq1_t qraw = (cq1_t)(uintptr_t)(a.qraw + (size_t)qb * qplane);
+    const cq1_t qflags = (cq1_t)(uintptr_t)(a.qflags + (size_t)qb * a.nchunks);
+
+    const int ch_begin = split * a.chunks_per_split;
+    const int ch_end = min(a.nchunks, ch_begin + a.chunks_per_split);
+
+    uint32_t pv[ELEMS];
+    auto load_chunk = [&](int ch) -> int {
+        const int64_t k0 = (int64_t)ch * KC;
+        int unsafe = 0;
+        if (PK == P_DENSE) {
+#pragma unroll
+            for (int i = 0; i < ELEMS; ++i) {
+                int rl, kk;
+                if (ALONG_K) { kk = tid & (KC - 1); rl = (tid >> 5) + i * (WG_THREADS / KC); }
+                else { rl = tid & (ROWS - 1); kk = i * (WG_THREADS / ROWS) + (tid / ROWS); }
+                const int64_t r = row0 + rl, k = k0 + kk;
+                uint32_t v = 0;
+                if (r < a.R && k < a.K) v = f2u(pbase[r * a.p.sr + k * a.p.sk]);
+                pv[i] = v;
+                unsafe |= operand_unsafe(v) ? 1 : 0;
+            }
+        } else if (PK == P_PATCH) {
+            // ALONG_K: this thread's k is fixed for the chunk
+            const int kk = tid & (KC - 1);
+            const int64_t k = k0 + kk;
+            const bool kvalid = k < a.K;
+            const int c = (int)(k % a.p.C);
+            const int t = (int)(k / a.p.C);
+            const int fx = t % a.p.KW, fy = t / a.p.KW;
+#pragma unroll
+            for (int i = 0; i < ELEMS; ++i) {
+                const int rl = (tid >> 5) + i * (WG_THREADS / KC);
+                const int vy = rowinfo[rl * 3 + 1] + fy, vx = rowinfo[rl * 3 + 2] + fx;
+                uint32_t v = 0;
+                if (kvalid && (unsigned)vy < (unsigned)a.p.VH && (unsigned)vx < (unsigned)a.p.VW) {
+                    int sy_ = vy, sx_ = vx;
+                    bool on_grid = true;
+                    if (a.p.dy != 1 || a.p.dx != 1) {
+                        sy_ = vy / a.p.dy;
+                        sx_ = vx / a.p.dx;
+                        on_grid = (sy_ * a.p.dy == vy) && (sx_ * a.p.dx == vx);
+                    }
+                    if (on_grid) v = f2u(pbase[rowinfo[rl * 3 + 0] + (sy_ * a.p.SW + sx_) * a.p.C + c]);
+                }
+                pv[i] = v;
+                unsafe |= operand_unsafe(v) ? 1 : 0;
+            }
+        } else {  // P_GF, staged along r
+            const int rl = tid & (ROWS - 1);
+            const int roff = rowinfo[rl * 3 + 0], fy = rowinfo[rl * 3 + 1], fx = rowinfo[rl * 3 + 2];
+#pragma unroll
+            for (int i = 0; i < ELEMS; ++i) {
+                const int kk = i * (WG_THREADS / ROWS) + __builtin_amdgcn_readfirstlane(tid / ROWS);
+                const int64_t k = k0 + kk;
+                uint32_t v = 0;
+                if (k < a.K) {
+                    const int x = (int)(k % a.p.GW);
+                    const int64_t t = k / a.p.GW;
+                    const int y = (int)(t % a.p.GH);
+                    const int b = (int)(t / a.p.GH);
+                    const int iy0 = y * a.p.sy - a.p.pt, ix0 = x * a.p.sx - a.p.pl;
+                    const int iy = iy0 + fy, ix = ix0 + fx;
+                    if ((unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
+                        v = f2u(pbase[((int64_t)(b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + roff]);
+                }
+                pv[i] = v;
+                unsafe |= operand_unsafe(v) ? 1 : 0;
+            }
+        }
+        return unsafe;
+    };
+    auto store_chunk = [&]() {
+#pragma unroll
+        for (int i = 0; i < ELEMS; ++i) {
+            int rl, kk;
+            if (ALONG_K) { kk = tid & (KC - 1); rl = (tid >> 5) + i * (WG_THREADS / KC); }
+            else { rl = tid & (ROWS - 1); kk = i * (WG_THREADS / ROWS) + (tid / ROWS); }
+            Pt[kk * RS + rl] = pv[i];
+        }
+    };
+
+    float acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[j] = 0.0f;
+
+    int unsafe = 0;
+    if (ch_begin < ch_end) unsafe = load_chunk(ch_begin);
+    const int lrow = wr * 64 + lane;
+    const int mshift = 23 - m;
+
+    for (int ch = ch_begin; ch < ch_end; ++ch) {
+        __syncthreads();  // every wave is done with the previous chunk's tile
+        store_chunk();
+        const int p_unsafe = __syncthreads_or(unsafe);
+        if (ch + 1 < ch_end) unsafe = load_chunk(ch + 1);  // in flight during the MACs below
+        if (!active) continue;
+        const uint32_t q_unsafe = qflags[ch];
+        const size_t qoff = (size_t)ch * KC * a.Jp + j0;
+        if (!(p_unsafe | q_unsafe)) {
+            cq2_t qrow = qd + qoff;
+#pragma unroll 4
+            for (int kk = 0; kk < KC; ++kk) {
+                const uint32_t raw = Pt[kk * RS + lrow];
+                const float ta = u2f(raw & 0xff800000u);
+                const uint32_t ia = (raw & 0x7fffffu) >> mshift;
+                uint32_t L[TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) L[j] = lut_s[qrow[j].y + ia];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const float t = u2f(qrow[j].x) * ta;
+                    const float f = u2f((L[j] << 16) + 0x3f800000u);
+                    acc[j] = __builtin_fmaf(t, f, acc[j]);
+                }
+                qrow += a.Jp;
+            }
+        } else {
+            cq1_t qrow = qraw + qoff;
+            for (int kk = 0; kk < KC; ++kk) {
+                const uint32_t raw = Pt[kk * RS + lrow];
+                const uint32_t ia = (raw & 0x7fffffu) >> mshift;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const uint32_t qr = qrow[j];
+                    const uint32_t e16 = (uint32_t)lut_s[(((qr & 0x7fffffu) >> mshift) << m) + ia] << 16;
+                    acc[j] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
+                }
+                qrow += a.Jp;
+            }
+        }
+    }
+
+    const int64_t r = row0 + lrow;
+    if (!active) return;
+    if (a.nsplit == 1) {
+        if (r < a.R) {
+            float *o = a.out + (int64_t)bz * a.out_batch_stride + r * a.so_r;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = acc[j];
+        }
+    } else {
+        float *o = a.partial + (((size_t)split * a.batch + bz) * a.Rp + r) * a.Jp + j0;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) o[j] = acc[j];
+    }
+}
+
+// sums the split partials in ascending split order (deterministic)
+struct RArgs {
+    const float *partial;
+    float *out;
+    int64_t R, J, Rp, so_r, so_j, out_batch_stride;
+    int Jp, nsplit, batch;
+};
+
+__global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
+{
+    const int64_t idx = (int64_t)blockIdx.x * WG_THREADS + threadIdx.x;
+    const int bz = blockIdx.y;
+    if (idx >= a.R * a.J) return;
+    const int64_t r = idx / a.J, j = idx - r * a.J;
+    float s = 0.0f;
+    for (int sp = 0; sp < a.nsplit; ++sp)
+        s += a.partial[(((size_t)sp * a.batch + bz) * a.Rp + r) * a.Jp + j];
+    a.out[(int64_t)bz * a.out_batch_stride + r * a.so_r + j * a.so_j] = s;
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct Plan {
+    int TN, WR, Jp, nchunks, nsplit, chunks_per_split;
+    int64_t Rp;
+    size_t off_qd, off_qraw, off_flags, off_partial, total;
+};
+
+static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
+{
+    Plan pl{};
+    pl.TN = J >= 9 ? 16 : J >= 5 ? 8 : J >= 3 ? 4 : (int)std::max<int64_t>(J, 1);
+    const int64_t jchunks = (J + pl.TN - 1) / pl.TN;
+    pl.WR = jchunks >= 2 ? 1 : 4;
+    pl.Jp = (int)((J + 15) / 16 * 16);
+    pl.nchunks = (int)((K + KC - 1) / KC);
+    const int rows = 64 * pl.WR;
+    pl.Rp = (R + rows - 1) / rows * rows;
+    const int64_t waves = ((R + 63) / 64) * jchunks * batch;
+    pl.nsplit = 1;
+    if (g_split_k.load() && waves < TARGET_WAVES / 2 && pl.nchunks > 1) {
+        int64_t want = (TARGET_WAVES + waves - 1) / waves;
+        pl.nsplit = (int)std::min<int64_t>(want, pl.nchunks);
+    }
+    pl.chunks_per_split = (pl.nchunks + pl.nsplit - 1) / pl.nsplit;
+    pl.nsplit = (pl.nchunks + pl.chunks_per_split - 1) / std::max(pl.chunks_per_split, 1);
+    if (pl.nchunks == 0) { pl.nsplit = 1; pl.chunks_per_split = 0; }
+    const size_t plane = (size_t)pl.nchunks * KC * pl.Jp;
+    size_t off = 0;
+    pl.off_qd = off;      off = align256(off + (size_t)q_batches * plane * sizeof(uint2));
+    pl.off_qraw = off;    off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
+    pl.off_flags = off;   off = align256(off + (size_t)q_batches * std::max(pl.nchunks, 1) * sizeof(uint32_t));
+    pl.off_partial = off;
+    if (pl.nsplit > 1) off = align256(off + (size_t)pl.nsplit * batch * pl.Rp * pl.Jp * sizeof(float));
+    pl.total = off;
+    return pl;
+}
+
+size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
+{
+    if (R <= 0 || J <= 0 || K <= 0 || batch <= 0) return 0;
+    return make_plan(R, J, K, batch, q_batches).total;
+}
+
+template <int TN, int WR>
+static void launch_variant(const KArgs &ka, dim3 grid, hipStream_t stream)
+{
+    const bool along_k = ka.p.kind == P_PATCH || (ka.p.kind == P_DENSE && ka.p.sk == 1 && ka.p.sr != 1);
+    if (ka.p.kind == P_DENSE) {
+        if (along_k) lutgemm_kernel<TN, WR, P_DENSE, true><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else lutgemm_kernel<TN, WR, P_DENSE, false><<<grid, WG_THREADS, 0, stream>>>(ka);
+    } else if (ka.p.kind == P_PATCH) {
+        lutgemm_kernel<TN, WR, P_PATCH, true><<<grid, WG_THREADS, 0, stream>>>(ka);
+    } else {
+        lutgemm_kernel<TN, WR, P_GF, false><<<grid, WG_THREADS, 0, stream>>>(ka);
+    }
+}
+
+int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream)
+{
+    if (d.R < 0 || d.J < 0 || d.K < 0 || d.batch < 0) return fail(AMSIM_ERR_INVALID, "negative GEMM extent");
+    if (d.R == 0 || d.J == 0 || d.batch == 0) return AMSIM_OK;
+    if (lut.m > 7 || lut.img_ab == nullptr)
+        return fail(AMSIM_ERR_UNSUPPORTED, "GEMM path needs a byte LUT image (mantissa width <= 7)");
+    if (d.K == 0) {
+        // empty reduction: the output is all zeros (matmulam.cc:154-160)
+        RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch};
+        dim3 grid((unsigned)((d.R * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
+        splitk_reduce_kernel<<<grid, WG_THREADS, 0, stream>>>(ra);
+        AMSIM_HIP_CHECK(hipGetLastError());
+        return AMSIM_OK;
+    }
+    if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
+        return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
+    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches);
+    if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < pl.total)
+        return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
+                                             std::to_string(pl.total) + " bytes");
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+
+    QArgs qa{};
+    qa.q = d.q;
+    qa.K = d.K; qa.J = d.J; qa.Jp = pl.Jp; qa.nchunks = pl.nchunks; qa.m = lut.m;
+    qa.qd = reinterpret_cast<uint2 *>(ws + pl.off_qd);
+    qa.qraw = reinterpret_cast<uint32_t *>(ws + pl.off_qraw);
+    qa.qflags = reinterpret_cast<uint32_t *>(ws + pl.off_flags);
+    q_prepass_kernel<<<dim3(pl.nchunks, d.q.batches), WG_THREADS, 0, stream>>>(qa);
+    AMSIM_HIP_CHECK(hipGetLastError());
+
+    KArgs ka{};
+    ka.p = d.p;
+    ka.lut_img = d.lane_first ? lut.img_ba : lut.img_ab;
+    ka.lut_bytes = (int)(((size_t)1 << (2 * lut.m)) + 15) / 16 * 16;
+    ka.m = lut.m;
+    ka.lane_first = d.lane_first ? 1 : 0;
+    ka.qd = qa.qd; ka.qraw = qa.qraw; ka.qflags = qa.qflags;
+    ka.q_batches = d.q.batches;
+    ka.R = d.R; ka.J = d.J; ka.K = d.K;
+    ka.Jp = pl.Jp; ka.nchunks = pl.nchunks; ka.nsplit = pl.nsplit; ka.chunks_per_split = pl.chunks_per_split;
+    ka.out = d.out; ka.so_r = d.so_r; ka.so_j = d.so_j; ka.out_batch_stride = d.out_batch_stride;
+    ka.partial = reinterpret_cast<float *>(ws + pl.off_partial);
+    ka.Rp = pl.Rp;
+    ka.batch = d.batch;
+
+    const int rows = 64 * pl.WR, wc = 4 / pl.WR;
+    const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;
+    const int64_t gz = (int64_t)d.batch * pl.nsplit;
+    if (gz > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch x split-K exceeds the grid limit");
+    dim3 grid((unsigned)(pl.Rp / rows), (unsigned)((jchunks + wc - 1) / wc), (unsigned)gz);
+    if (grid.y > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "uniform dimension exceeds the grid limit");
+    switch (pl.TN) {
+    case 16:
+        if (pl.WR == 1) launch_variant<16, 1>(ka, grid, stream);
+        else launch_variant<16, 4>(ka, grid, stream);
+        break;
+    case 8: launch_variant<8, 4>(ka, grid, stream); break;
+    case 4: launch_variant<4, 4>(ka, grid, stream); break;
+    case 2: launch_variant<2, 4>(ka, grid, stream); break;
+    default: launch_variant<1, 4>(ka, grid, stream); break;
+    }
+    AMSIM_HIP_CHECK(hipGetLastError());
+
+    if (pl.nsplit > 1) {
+        RArgs ra{ka.partial, d.out, d.R, d.J, pl.Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp, pl.nsplit, d.batch};
+        dim3 rgrid((unsigned)((d.R * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
+        splitk_reduce_kernel<<<rgrid, WG_THREADS, 0, stream>>>(ra);
+        AMSIM_HIP_CHECK(hipGetLastError());
+    }
+    return AMSIM_OK;
+}
+
+// ---------------------------------------------------------------------------
+// elementwise product (test hook)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(WG_THREADS) void mul_kernel(const uint32_t *lut32, int m, const float *a,
+                                                         const float *b, float *out, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * WG_THREADS + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * WG_THREADS;
+    for (; i < n; i += stride) {
+        const uint32_t at = f2u(a[i]), bt = f2u(b[i]);
+        const uint32_t ma = (at & 0x7fffffu) >> (23 - m), mb = (bt & 0x7fffffu) >> (23 - m);
+        out[i] = am_exact(at, bt, lut32[(ma << m) | mb]);
+    }
+}
+
+int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream)
+{
+    if (n == 0) return AMSIM_OK;
+    const unsigned blocks = (unsigned)std::min<size_t>((n + WG_THREADS - 1) / WG_THREADS, 65535u * 16u);
+    mul_kernel<<<blocks, WG_THREADS, 0, stream>>>(lut.lut32, lut.m, a, b, out, n);
+    AMSIM_HIP_CHECK(hipGetLastError());
+    return AMSIM_OK;
+}
+
+void set_split_k(int mode) { g_split_k.store(mode ? 1 : 0); }
+
+}  // namespace amsim

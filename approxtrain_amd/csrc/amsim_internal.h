@@ -1,0 +1,100 @@
+// Internal declarations shared by the amsim translation units (not installed).
+#ifndef AMSIM_INTERNAL_H_
+#define AMSIM_INTERNAL_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <string>
+
+#include "amsim.h"
+
+namespace amsim {
+
+// ---- error plumbing ---------------------------------------------------------
+void set_error(const std::string &msg);
+int fail(int status, const std::string &msg);
+#define AMSIM_HIP_CHECK(expr)                                                                       \
+    do {                                                                                            \
+        hipError_t e_ = (expr);                                                                     \
+        if (e_ != hipSuccess)                                                                       \
+            return ::amsim::fail(AMSIM_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)); \
+    } while (0)
+
+// ---- LUT handle -------------------------------------------------------------
+// Device images of one mantissa-product table.
+//   img_ab[(ma << m) | mb]  one byte per entry: carry << 7 | mantissa << (7 - m)
+//   img_ba[(mb << m) | ma]  the same table transposed
+// (m <= 7 only; both are padded to a multiple of 16 bytes), and
+//   lut32[(ma << m) | mb]   carry << 23 | mantissa << (23 - m)   (every m)
+struct Lut {
+    int m = 0;
+    int device = 0;
+    size_t entries = 0;
+    uint8_t *img_ab = nullptr;
+    uint8_t *img_ba = nullptr;
+    uint32_t *lut32 = nullptr;
+    uint32_t *lut32_t = nullptr;  // transposed 32-bit table (m > 7 path)
+};
+
+}  // namespace amsim
+
+struct amsim_lut {
+    amsim::Lut l;
+};
+
+namespace amsim {
+
+// ---- the GEMM engine ----------------------------------------------------------
+// out(r, j) = sum_k P(p(r, k), q(k, j)).  r is the dimension spread over the
+// lanes of a wavefront ("lane operand" p), j the dimension kept wave-uniform
+// ("uniform operand" q, pre-decoded into the workspace and read through the
+// scalar cache).  lane_first tells which operand indexes the LUT row (ma).
+enum PKind { P_DENSE = 0, P_PATCH = 1, P_GF = 2 };
+enum QKind { Q_DENSE = 0, Q_FLIP = 1 };
+
+struct PDesc {
+    int kind = P_DENSE;
+    const float *base = nullptr;
+    int64_t batch_stride = 0;
+    // P_DENSE: element (r, k) at base[r * sr + k * sk]
+    int64_t sr = 0, sk = 0;
+    // P_PATCH: r = (b, y, x) over [B, GH, GW], k = (fy, fx, c) over [KH, KW, C];
+    //          virtual source pixel (y*sy - pt + fy, x*sx - pl + fx) on a grid of
+    //          VH x VW that holds the real [B, SH, SW, C] source at multiples of
+    //          (dy, dx) and zeros elsewhere.
+    // P_GF:    r = (fy, fx, c) over [KH, KW, C], k = (b, y, x) over [B, GH, GW];
+    //          source pixel (y*sy - pt + fy, x*sx - pl + fx) of [B, SH, SW, C].
+    int B = 0, GH = 0, GW = 0, KH = 0, KW = 0, C = 0;
+    int sy = 1, sx = 1, pt = 0, pl = 0, dy = 1, dx = 1, VH = 0, VW = 0, SH = 0, SW = 0;
+};
+
+struct QDesc {
+    int kind = Q_DENSE;
+    const float *base = nullptr;
+    int64_t batch_stride = 0;
+    int batches = 1;  // 1 = shared by every batch item
+    // Q_DENSE: element (k, j) at base[k * sk + j * sj]
+    int64_t sk = 0, sj = 0;
+    // Q_FLIP: k = (fy, fx, oc), j = ic of an HWIO filter [KH, KW, IC, OC]:
+    //         base[((KH-1-fy) * KW + (KW-1-fx)) * IC * OC + ic * OC + oc]
+    int KH = 0, KW = 0, IC = 0, OC = 0;
+};
+
+struct GemmDesc {
+    PDesc p;
+    QDesc q;
+    int64_t R = 0, J = 0, K = 0;
+    int batch = 1;
+    float *out = nullptr;
+    int64_t so_r = 0, so_j = 0, out_batch_stride = 0;
+    bool lane_first = true;
+};
+
+size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
+int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream);
+
+int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream);
+
+}  // namespace amsim
+#endif

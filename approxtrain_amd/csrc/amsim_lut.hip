@@ -1,0 +1,205 @@
+// LUT handle: host-side loading (the counterpart of approx_mul_lut.h:15-46) and
+// the device images the kernels read (the counterpart of the cudaMalloc +
+// texture object of cuda/approx_mul_lut.cu:24-48).
+#include "amsim_internal.h"
+
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <vector>
+
+namespace amsim {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string &msg) { g_last_error = msg; }
+
+int fail(int status, const std::string &msg)
+{
+    g_last_error = msg;
+    return status;
+}
+
+const std::string &last_error() { return g_last_error; }
+
+// entries: one (carry, mantissa) pair per (ma, mb), mantissa in m bits
+static int build_images(int m, const std::vector<uint8_t> &carry, const std::vector<uint32_t> &mant, Lut *out)
+{
+    const size_t n = (size_t)1 << m, total = n * n;
+    std::vector<uint32_t> l32(total), l32t(total);
+    for (size_t i = 0; i < n; ++i)
+        for (size_t j = 0; j < n; ++j) {
+            const uint32_t v = ((uint32_t)carry[i * n + j] << 23) | (mant[i * n + j] << (23 - m));
+            l32[i * n + j] = v;
+            l32t[j * n + i] = v;
+        }
+    Lut l;
+    l.m = m;
+    l.entries = total;
+    AMSIM_HIP_CHECK(hipGetDevice(&l.device));
+    AMSIM_HIP_CHECK(hipMalloc(&l.lut32, total * 4));
+    AMSIM_HIP_CHECK(hipMemcpy(l.lut32, l32.data(), total * 4, hipMemcpyHostToDevice));
+    AMSIM_HIP_CHECK(hipMalloc(&l.lut32_t, total * 4));
+    AMSIM_HIP_CHECK(hipMemcpy(l.lut32_t, l32t.data(), total * 4, hipMemcpyHostToDevice));
+    if (m <= 7) {
+        const size_t padded = (total + 15) / 16 * 16;
+        std::vector<uint8_t> ab(padded, 0), ba(padded, 0);
+        for (size_t i = 0; i < n; ++i)
+            for (size_t j = 0; j < n; ++j) {
+                const uint8_t b = (uint8_t)((carry[i * n + j] << 7) | (mant[i * n + j] << (7 - m)));
+                ab[i * n + j] = b;
+                ba[j * n + i] = b;
+            }
+        AMSIM_HIP_CHECK(hipMalloc(&l.img_ab, padded));
+        AMSIM_HIP_CHECK(hipMemcpy(l.img_ab, ab.data(), padded, hipMemcpyHostToDevice));
+        AMSIM_HIP_CHECK(hipMalloc(&l.img_ba, padded));
+        AMSIM_HIP_CHECK(hipMemcpy(l.img_ba, ba.data(), padded, hipMemcpyHostToDevice));
+    }
+    *out = l;
+    return AMSIM_OK;
+}
+
+int lut_from_entries(const void *entries, size_t n_bytes, int m, int entry_bytes, Lut *out)
+{
+    if (entries == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT entries");
+    if (entry_bytes != 1 && entry_bytes != 4) return fail(AMSIM_ERR_LUT_FORMAT, "entry_bytes must be 1 or 4");
+    if (m < 1 || (entry_bytes == 1 && m > 7) || m > 11)
+        return fail(AMSIM_ERR_LUT_FORMAT, "mantissa width " + std::to_string(m) + " unsupported for " +
+                                              std::to_string(entry_bytes) + "-byte entries");
+    const size_t total = (size_t)1 << (2 * m);
+    if (n_bytes < total * entry_bytes)
+        return fail(AMSIM_ERR_LUT_FORMAT, "LUT holds " + std::to_string(n_bytes) + " bytes, needs " +
+                                              std::to_string(total * entry_bytes));
+    std::vector<uint8_t> carry(total);
+    std::vector<uint32_t> mant(total);
+    if (entry_bytes == 1) {
+        // lut/lut_gen.cc:114-121: carry << 7 | mantissa (m bits, right-aligned)
+        const uint8_t *e = static_cast<const uint8_t *>(entries);
+        for (size_t i = 0; i < total; ++i) {
+            carry[i] = e[i] >> 7;
+            mant[i] = (e[i] & 0x7fu) & ((1u << m) - 1u);
+        }
+    } else {
+        // lut/AMsimulator.inl:18-20: bit 31 = carry, bits 22..0 = mantissa in place
+        const uint32_t *e = static_cast<const uint32_t *>(entries);
+        for (size_t i = 0; i < total; ++i) {
+            carry[i] = (uint8_t)(e[i] >> 31);
+            mant[i] = (e[i] & 0x7fffffu) >> (23 - m);
+        }
+    }
+    return build_images(m, carry, mant, out);
+}
+
+void lut_free(Lut &l)
+{
+    if (l.img_ab) (void)hipFree(l.img_ab);
+    if (l.img_ba) (void)hipFree(l.img_ba);
+    if (l.lut32) (void)hipFree(l.lut32);
+    if (l.lut32_t) (void)hipFree(l.lut32_t);
+    l = Lut{};
+}
+
+// approx_mul_lut.h:22-25: the width is the decimal number between the last
+// '_' and the last '.' of the file name.
+int parse_width_from_name(const std::string &path, int *m)
+{
+    const size_t us = path.find_last_of('_'), dot = path.find_last_of('.');
+    if (us == std::string::npos || dot == std::string::npos || dot <= us + 1)
+        return fail(AMSIM_ERR_LUT_FORMAT, "LUT file name '" + path + "' lacks the _<width>.<ext> suffix");
+    const std::string w = path.substr(us + 1, dot - us - 1);
+    for (char c : w)
+        if (c < '0' || c > '9')
+            return fail(AMSIM_ERR_LUT_FORMAT, "LUT file name '" + path + "': width '" + w + "' is not a number");
+    if (w.size() > 3) return fail(AMSIM_ERR_LUT_FORMAT, "LUT file name '" + path + "': width out of range");
+    *m = std::stoi(w);
+    return AMSIM_OK;
+}
+
+}  // namespace amsim
+
+using namespace amsim;
+
+extern "C" {
+
+const char *amsim_last_error(void) { return amsim::last_error().c_str(); }
+
+const char *amsim_status_string(int status)
+{
+    switch (status) {
+    case AMSIM_OK: return "ok";
+    case AMSIM_ERR_INVALID: return "invalid argument";
+    case AMSIM_ERR_IO: return "LUT file I/O error";
+    case AMSIM_ERR_LUT_FORMAT: return "bad LUT format";
+    case AMSIM_ERR_HIP: return "HIP runtime error";
+    case AMSIM_ERR_WORKSPACE: return "workspace missing or too small";
+    case AMSIM_ERR_UNSUPPORTED: return "unsupported";
+    default: return "unknown status";
+    }
+}
+
+int amsim_device_info(char *arch, size_t arch_len, int *compute_units)
+{
+    int dev = 0;
+    AMSIM_HIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    AMSIM_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+    if (arch && arch_len) {
+        std::snprintf(arch, arch_len, "%s", prop.gcnArchName);
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    return AMSIM_OK;
+}
+
+int amsim_lut_create(const void *entries, size_t n_bytes, int mant_width, int entry_bytes, amsim_lut_t *out)
+{
+    if (out == nullptr) return fail(AMSIM_ERR_INVALID, "null output handle");
+    *out = nullptr;
+    Lut l;
+    int rc = lut_from_entries(entries, n_bytes, mant_width, entry_bytes, &l);
+    if (rc != AMSIM_OK) return rc;
+    *out = new amsim_lut{l};
+    return AMSIM_OK;
+}
+
+int amsim_lut_load_file(const char *path, amsim_lut_t *out)
+{
+    if (out == nullptr) return fail(AMSIM_ERR_INVALID, "null output handle");
+    *out = nullptr;
+    if (path == nullptr || *path == '\0') return fail(AMSIM_ERR_INVALID, "no mant lut file name given");
+    int m = 0;
+    int rc = parse_width_from_name(path, &m);
+    if (rc != AMSIM_OK) return rc;
+    if (m < 1 || m > 7)
+        return fail(AMSIM_ERR_LUT_FORMAT, "LUT files hold one byte per entry: mantissa width must be 1..7, got " +
+                                              std::to_string(m));
+    std::ifstream file(path, std::ios::in | std::ios::binary);
+    if (!file.is_open() || file.fail()) return fail(AMSIM_ERR_IO, std::string("lut file open failed: ") + path);
+    const size_t total = (size_t)1 << (2 * m);
+    std::vector<uint8_t> bytes(total);
+    file.read(reinterpret_cast<char *>(bytes.data()), (std::streamsize)total);
+    if ((size_t)file.gcount() != total)
+        return fail(AMSIM_ERR_LUT_FORMAT, std::string("lut file too short: ") + path);
+    return amsim_lut_create(bytes.data(), total, m, 1, out);
+}
+
+int amsim_lut_destroy(amsim_lut_t lut)
+{
+    if (lut == nullptr) return AMSIM_OK;
+    lut_free(lut->l);
+    delete lut;
+    return AMSIM_OK;
+}
+
+int amsim_lut_mant_width(amsim_lut_t lut) { return lut ? lut->l.m : -1; }
+
+int amsim_lut_params(amsim_lut_t lut, uint32_t *mant_mask, int *a_shift, int *b_shift)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    const int m = lut->l.m;
+    if (mant_mask) *mant_mask = ((1u << m) - 1u) << (23 - m);
+    if (a_shift) *a_shift = 23 - 2 * m;
+    if (b_shift) *b_shift = 23 - m;
+    return AMSIM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,167 @@
+/*
+ * amsim.h -- C ABI of the MI355X (gfx950) approximate-multiplier simulator.
+ *
+ * This is the drop-in seam underneath ApproxTrain's custom-op surface: each
+ * entry point replaces one of the reference's device functors / kernels, takes
+ * plain device pointers, sizes and a HIP stream, and returns a status code
+ * (the reference prints and calls exit(); cuda/error.cuh:19-27).
+ *
+ * Conventions
+ *   - all tensors are FP32 in device memory; NHWC activations, HWIO filters,
+ *     row-major matrices (as in the reference);
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream); calls
+ *     are stream-ordered and never synchronise the device (the reference calls
+ *     cudaDeviceSynchronize after every launch);
+ *   - the library allocates device memory only in amsim_lut_create /
+ *     amsim_lut_load_file; per-call scratch comes from the caller as
+ *     `workspace` (size from the matching *_workspace_bytes query, 256-byte
+ *     aligned), the way the reference's OpKernels allocate their im2col /
+ *     rsfilter temporaries and hand them to the functor;
+ *   - the approximate product follows the C functional models
+ *     (lut/FPmultMBM_fast16.inl:45-134, lut/Mitchell_16.inl:44-129) bit for
+ *     bit on the whole FP32 domain, given the matching LUT;
+ *   - every output element is one FP32 accumulation chain in ascending
+ *     reduction index when the reduction is not split; the filter gradient and
+ *     small problems split the reduction deterministically (fixed chunking,
+ *     fixed summation order), so results are reproducible run to run.
+ */
+#ifndef AMSIM_H_
+#define AMSIM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AMSIM_OK 0
+#define AMSIM_ERR_INVALID 1     /* bad argument / shape mismatch (OP_REQUIRES InvalidArgument in the reference) */
+#define AMSIM_ERR_IO 2          /* LUT file missing or unreadable (exit(1) in approx_mul_lut.h:31-40) */
+#define AMSIM_ERR_LUT_FORMAT 3  /* file name without _<m>.bin suffix, unsupported width, short file */
+#define AMSIM_ERR_HIP 4         /* a HIP runtime call failed */
+#define AMSIM_ERR_WORKSPACE 5   /* workspace missing, misaligned or too small */
+#define AMSIM_ERR_UNSUPPORTED 6
+
+/* padding attr values, numerically equal to tensorflow::Padding (convam.cc:552 tests `padding == 1`) */
+#define AMSIM_PADDING_VALID 1
+#define AMSIM_PADDING_SAME 2
+
+typedef struct amsim_lut *amsim_lut_t;
+
+const char *amsim_status_string(int status);
+/* message of the last failing call on this thread ("" if none) */
+const char *amsim_last_error(void);
+/* "gfx950" etc. of the current device, and the number of compute units */
+int amsim_device_info(char *arch, size_t arch_len, int *compute_units);
+
+/* ---- LUT handle: replaces approx_mul_lut<GPUDevice>
+ *      (approx_mul_lut.h:7-80, cuda/approx_mul_lut.cu:24-53) -------------------
+ * amsim_lut_load_file parses the mantissa width from the file name between the
+ * last '_' and the last '.' (approx_mul_lut.h:22-25) and reads 2^(2m) entries:
+ * 1 byte each (carry<<7 | mantissa, lut/lut_gen.cc:114-121) for m <= 7.
+ * amsim_lut_create takes the entries from host memory; entry_bytes is 1
+ * (layout above, m <= 7) or 4 (legacy layout of lut/AMsimulator.inl:18-20:
+ * bit 31 = carry, bits 22..0 = mantissa in place; m <= 11). */
+int amsim_lut_load_file(const char *path, amsim_lut_t *out);
+int amsim_lut_create(const void *entries, size_t n_bytes, int mant_width, int entry_bytes, amsim_lut_t *out);
+int amsim_lut_destroy(amsim_lut_t lut);
+int amsim_lut_mant_width(amsim_lut_t lut);
+/* the derived fields of approx_mul_lut.h:26-28 */
+int amsim_lut_params(amsim_lut_t lut, uint32_t *mant_mask, int *a_shift, int *b_shift);
+
+/* ---- elementwise product (test hook): the device function AMsimulator
+ *      (cuda/AMsimulator.inl:13-36) with the functional models' semantics ---- */
+int amsim_mul_f32(amsim_lut_t lut, const float *a, const float *b, float *out, size_t n, void *stream);
+
+/* ---- GEMM: replaces gemm<float> (cuda/gemm.cu:17-58) ------------------------
+ * C[i][j] = sum_k P(opA(i,k), opB(k,j)); opA is M x K (A[i*lda+k], or
+ * A[k*lda+i] if transA), opB is K x N.  swap_operands feeds the LUT as
+ * P(B element, A element) (denseam_kernel.cu:93).  batch > 1 runs a strided
+ * batch (stride 0 broadcasts an operand), replacing the per-item launch loop
+ * of cuda/matmulam_kernel.cu:30-98. */
+size_t amsim_gemm_workspace_bytes(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch);
+int amsim_gemm_f32(amsim_lut_t lut, int transA, int transB, int swap_operands, int64_t M, int64_t N,
+                   int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                   int64_t ldc, int64_t batch, int64_t strideA, int64_t strideB, int64_t strideC,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- convolution functors ----------------------------------------------------
+ * Argument names and order follow convam.h:71-104; the im2col / rsfilter
+ * temporaries of the reference are replaced by `workspace`. */
+
+/* ConvamFunctor<GPUDevice,float>::operator() (convam.h:71-79, cuda_kernel.cu:181-321) */
+size_t amsim_convam_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth, int filter_rows,
+                                    int filter_cols, int in_depth);
+int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
+                     int out_cols, int out_depth, int stride_cols, int stride_rows, int filter_left_offset,
+                     int filter_top_offset, int filter_rows, int filter_cols, int in_depth, int input_cols,
+                     int input_rows, const float *filter, void *workspace, size_t workspace_bytes,
+                     void *stream);
+
+/* ConvamInputGradFunctor<GPUDevice,float>::operator() (convam.h:84-92,
+ * cuda_kernel.cu:590-657).  pad_top/pad_left are the BACK pads
+ * filter - 1 - forward_pad (convam.cc:1083-1084); hole_grad_* is the
+ * stride-dilated gradient extent (convam.cc:1066-1067). */
+size_t amsim_convam_input_grad_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
+                                               int filter_rows, int filter_cols, int out_depth);
+int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_grad_width, int hole_grad_height,
+                                int pad_top, int pad_left, const float *filter, int filter_rows,
+                                int filter_cols, int out_depth, int stride_rows, int stride_cols, int batch,
+                                int input_rows, int input_cols, int in_depth, float *output, int out_rows,
+                                int out_cols, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ConvamFilterGradFunctor<GPUDevice,float>::operator() (convam.h:97-104,
+ * cuda_kernel.cu:431-461) */
+size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth,
+                                                int filter_rows, int filter_cols, int in_depth);
+int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const float *grad, int input_rows,
+                                 int input_cols, int batch, int in_depth, int out_cols, int out_rows,
+                                 int out_depth, int filter_left_offset, int filter_top_offset, int stride_rows,
+                                 int stride_cols, int filter_cols, int filter_rows, float *output,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- dense functors (denseam.h:9-27, cuda/denseam_kernel.cu:98-145) ---------- */
+size_t amsim_denseam_workspace_bytes(int batch, int units, int input_width);
+/* DenseamFunctor: output[batch][units] = inputs[batch][input_width] . weights[input_width][units] */
+int amsim_denseam_f32(amsim_lut_t lut, const float *inputs, const float *weights, float *output, int batch,
+                      int units, int input_width, void *workspace, size_t workspace_bytes, void *stream);
+/* DenseamWeightGradFunctor: grad_weights[k][j] = sum_i P(input[i][k], grads[i][j]) */
+int amsim_denseam_weight_grad_f32(amsim_lut_t lut, const float *input, const float *grads, float *output,
+                                  int batch, int units, int input_width, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+/* DenseamInputGradFunctor: grad_inputs[i][k] = sum_j P(weight[k][j], grads[i][j]) */
+int amsim_denseam_input_grad_f32(amsim_lut_t lut, const float *weight, const float *grads, float *output,
+                                 int batch, int units, int input_width, void *workspace,
+                                 size_t workspace_bytes, void *stream);
+
+/* ---- LaunchMatMul<GPUDevice,float> (matmulam.h:12-17, matmulam_kernel.cu:12-99)
+ * batch_a / batch_b: 0 for a rank-2 operand, else its leading dimension; a
+ * batch of 1 broadcasts (matmulam.cc:86-147). */
+size_t amsim_matmulam_workspace_bytes(int batch_a, int batch_b, int row_a, int col_a, int row_b, int col_b);
+int amsim_matmulam_f32(amsim_lut_t lut, const float *a, const float *b, int batch_a, int batch_b, int row_a,
+                       int col_a, int row_b, int col_b, float *out, void *workspace, size_t workspace_bytes,
+                       void *stream);
+
+/* ---- op-level host logic (what the OpKernel::Compute bodies derive) ----------
+ * TensorFlow 2.3 GetWindowedOutputSizeVerbose for dilation 1 as used at
+ * convam.cc:382-387, 553-572, 1071-1084: output extent and leading pad. */
+int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, int *out_size, int *pad_before);
+
+/* ---- knobs and measurement helpers (no counterpart in the reference) ----------
+ * amsim_set_split_k(0) forces every reduction to stay one sequential chain per
+ * output (bit-identical to a sequential CPU loop); 1 (default) lets problems
+ * with few outputs split the reduction across workgroups. */
+int amsim_set_split_k(int mode);
+/* Micro-kernels that measure, on the current device, the VALU issue rate
+ * (kind 0: independent FP32 FMAs) and the LDS gather rate (kinds 1..6: u8 /
+ * u16 / b32 reads, lanes inside one 128-element row or scattered).  Launches
+ * `reps` times on `stream`, timed with HIP events; `sink` is any device buffer
+ * of >= 256 floats. */
+int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream, float *sink,
+                     double *ms_per_launch, double *ops_per_launch);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AMSIM_H_ */

@@ -1,0 +1,200 @@
+"""LUT-multiply GEMM, dense and matmul entry points on the GPU (through the C
+ABI) against the CPU oracle on the same seeded inputs.
+
+Bars: with the reduction unsplit every output is one ascending-k FP32 chain,
+so results are BIT-EQUAL to the oracle; with split-K (small problems) they are
+within 1e-5 * sum_k |product| (the tolerance the task states)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu
+from tests.gpu_util import assert_close_sum_abs, asym_lut_u8, dev, host, lut32
+from tests.util import lut_path, small_ints
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import approxtrain_amd
+    from approxtrain_amd import functors
+    lib = approxtrain_amd.load_library()
+    yield functors
+    lib.amsim_set_split_k(1)
+
+
+def _set_split(mode):
+    import approxtrain_amd
+    approxtrain_amd.load_library().amsim_set_split_k(mode)
+
+
+def _ops(rng, M, N, K, ta, tb, relu=False):
+    A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+    B = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    if relu:
+        A = np.maximum(A, 0)
+    return A, B
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 16, 32), (100, 37, 77), (257, 300, 129), (1, 1, 1), (3, 130, 40),
+                                   (130, 3, 40), (65, 6, 150), (200, 1, 33), (128, 300, 784)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_bit_equal_when_unsplit(amd, M, N, K, ta, tb):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    rng = np.random.default_rng(M * 7 + N * 3 + K + ta * 2 + tb)
+    A, B = _ops(rng, M, N, K, ta, tb, relu=True)
+    lut = ApproxMulLut(lut_path("MBM", 7))
+    got = host(amd.gemm(lut, dev(A), dev(B), trans_a=bool(ta), trans_b=bool(tb)))
+    want = cpu.gemm(lut32("MBM", 7), 7, A, B, transA=ta, transB=tb)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("kind,m", [("MBM", 1), ("MBM", 3), ("MBM", 5), ("MIT", 1), ("MIT", 3), ("MIT", 5),
+                                    ("MIT", 7), ("ACC", 7)])
+def test_gemm_every_lut_width(amd, kind, m):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    rng = np.random.default_rng(50 + m)
+    A, B = _ops(rng, 150, 70, 96, 0, 0)
+    got = host(amd.gemm(ApproxMulLut(lut_path(kind, m)), dev(A), dev(B)))
+    want = cpu.gemm(lut32(kind, m), m, A, B)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("swap", [False, True])
+@pytest.mark.parametrize("M,N", [(90, 20), (20, 90)])  # both lane orientations
+def test_gemm_operand_order_with_asymmetric_lut(amd, swap, M, N):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    tab = asym_lut_u8(3)
+    lut = ApproxMulLut.from_entries(tab, 3)
+    rng = np.random.default_rng(61)
+    A, B = _ops(rng, M, N, 45, 0, 0)
+    got = host(amd.gemm(lut, dev(A), dev(B), swap_operands=swap))
+    want = cpu.gemm(cpu.expand_u8(tab, 3), 3, A, B, swap=swap)
+    other = cpu.gemm(cpu.expand_u8(tab, 3), 3, A, B, swap=not swap)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert not np.array_equal(want, other)
+
+
+def test_gemm_full_domain_operands_take_exact_path(amd):
+    """Subnormals, infinities, NaNs, huge and tiny magnitudes inside the
+    operands: the flagged chunks must reproduce the functional-model product."""
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    rng = np.random.default_rng(62)
+    M, N, K = 96, 40, 128
+    A = (rng.standard_normal((M, K)) * 2.0 ** rng.integers(-70, 70, (M, K))).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 2.0 ** rng.integers(-70, 70, (K, N))).astype(np.float32)
+    A[3, 5] = np.float32(1e-41); A[10, 40] = np.inf; A[20, 70] = np.nan; A[0, 0] = 0.0; A[50, 100] = -0.0
+    B[5, 3] = np.float32(-3e-40); B[64, 7] = -np.inf; B[33, 1] = np.float32(3e38); B[100, 2] = 0.0
+    got = host(amd.gemm(ApproxMulLut(lut_path("MBM", 7)), dev(A), dev(B)))
+    with np.errstate(all="ignore"):
+        want = cpu.gemm(lut32("MBM", 7), 7, A, B)
+    both_nan = np.isnan(got) & np.isnan(want)
+    assert ((got.view(np.uint32) == want.view(np.uint32)) | both_nan).all()
+    assert np.isnan(want).any() and np.isinf(want).any()
+
+
+def test_gemm_split_k_within_tolerance_and_deterministic(amd):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(1)
+    rng = np.random.default_rng(63)
+    A, B = _ops(rng, 128, 300, 784, 0, 0)
+    lut = ApproxMulLut(lut_path("MBM", 7))
+    got = host(amd.gemm(lut, dev(A), dev(B)))
+    again = host(amd.gemm(lut, dev(A), dev(B)))
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    want = cpu.gemm(lut32("MBM", 7), 7, A, B)
+    assert_close_sum_abs(got, want, cpu.gemm_abs(lut32("MBM", 7), 7, A, B))
+
+
+def test_gemm_exact_on_integers(amd):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(1)
+    rng = np.random.default_rng(64)
+    A, B = small_ints(rng, (200, 333)), small_ints(rng, (333, 50))
+    got = host(amd.gemm(ApproxMulLut(lut_path("ACC", 7)), dev(A), dev(B)))
+    assert np.array_equal(got.astype(np.int64), A.astype(np.int64) @ B.astype(np.int64))
+
+
+def test_gemm_strided_batch_and_broadcast(amd):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    rng = np.random.default_rng(65)
+    lut = ApproxMulLut(lut_path("MBM", 7))
+    L = lut32("MBM", 7)
+    A = rng.standard_normal((5, 70, 48)).astype(np.float32)
+    B = rng.standard_normal((5, 48, 33)).astype(np.float32)
+    got = host(amd.gemm(lut, dev(A), dev(B)))
+    for i in range(5):
+        assert np.array_equal(got[i].view(np.uint32), cpu.gemm(L, 7, A[i], B[i]).view(np.uint32))
+    got = host(amd.gemm(lut, dev(A), dev(B[0])))
+    for i in range(5):
+        assert np.array_equal(got[i].view(np.uint32), cpu.gemm(L, 7, A[i], B[0]).view(np.uint32))
+    got = host(amd.gemm(lut, dev(A[0]), dev(B), trans_b=False))
+    for i in range(5):
+        assert np.array_equal(got[i].view(np.uint32), cpu.gemm(L, 7, A[0], B[i]).view(np.uint32))
+
+
+@pytest.mark.parametrize("ba,bb", [(0, 0), (3, 3), (3, 1), (1, 3), (3, 0), (0, 3)])
+def test_matmulam_shape_cases(amd, ba, bb):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    rng = np.random.default_rng(66)
+    a = rng.standard_normal(((ba,) if ba else ()) + (40, 24)).astype(np.float32)
+    b = rng.standard_normal(((bb,) if bb else ()) + (24, 50)).astype(np.float32)
+    got = host(amd.matmulam(ApproxMulLut(lut_path("MIT", 7)), dev(a), dev(b)))
+    want = cpu.matmul(lut32("MIT", 7), 7, a, b)
+    assert got.shape == want.shape
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_matmulam_errors_and_empty(amd):
+    from approxtrain_amd import AmsimError, ApproxMulLut
+    lut = ApproxMulLut(lut_path("MIT", 7))
+    with pytest.raises(AmsimError):
+        amd.matmulam(lut, torch.zeros(2, 3, device="cuda"), torch.zeros(4, 5, device="cuda"))
+    with pytest.raises(AmsimError):
+        amd.matmulam(lut, torch.zeros(2, 2, 3, device="cuda"), torch.zeros(3, 3, 5, device="cuda"))
+    out = amd.matmulam(lut, torch.zeros(4, 0, device="cuda"), torch.zeros(0, 5, device="cuda"))
+    assert out.shape == (4, 5) and float(out.abs().sum()) == 0.0  # matmulam.cc:154-160
+    out = amd.matmulam(lut, torch.zeros(0, 3, device="cuda"), torch.zeros(3, 5, device="cuda"))
+    assert out.shape == (0, 5)
+
+
+def test_denseam_lenet300_first_layer(amd):
+    """denseam forward at LeNet-300-100's first layer: X[128,784] uniform[0,1),
+    W[784,300] Glorot-uniform, MBM_7; plus both gradients."""
+    from approxtrain_amd import ApproxMulLut
+    lut = ApproxMulLut(lut_path("MBM", 7))
+    L = lut32("MBM", 7)
+    x = np.random.default_rng(1).random((128, 784), dtype=np.float32)
+    lim = np.sqrt(6.0 / (784 + 300))
+    w = np.random.default_rng(2).uniform(-lim, lim, (784, 300)).astype(np.float32)
+    dy = (np.random.default_rng(3).standard_normal((128, 300)) * 0.1).astype(np.float32)
+    _set_split(0)
+    y = host(amd.denseam(lut, dev(x), dev(w)))
+    assert np.array_equal(y.view(np.uint32), cpu.dense_fwd(L, 7, x, w).view(np.uint32))
+    dx, dw = amd.denseam_grad(lut, dev(dy), dev(x), dev(w))
+    dx_ref, dw_ref = cpu.dense_grad(L, 7, dy, x, w)
+    assert np.array_equal(host(dx).view(np.uint32), dx_ref.view(np.uint32))
+    assert np.array_equal(host(dw).view(np.uint32), dw_ref.view(np.uint32))
+    _set_split(1)
+    y = host(amd.denseam(lut, dev(x), dev(w)))
+    assert_close_sum_abs(y, cpu.dense_fwd(L, 7, x, w), cpu.gemm_abs(L, 7, x, w))
+
+
+def test_dense_grad_operand_order(amd):
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    tab = asym_lut_u8(3)
+    lut = ApproxMulLut.from_entries(tab, 3)
+    rng = np.random.default_rng(67)
+    x, w, dy = (rng.standard_normal(s).astype(np.float32) for s in ((30, 50), (50, 40), (30, 40)))
+    dx, dw = amd.denseam_grad(lut, dev(dy), dev(x), dev(w))
+    dx_ref, dw_ref = cpu.dense_grad(cpu.expand_u8(tab, 3), 3, dy, x, w)
+    assert np.array_equal(host(dx).view(np.uint32), dx_ref.view(np.uint32))
+    assert np.array_equal(host(dw).view(np.uint32), dw_ref.view(np.uint32))

@@ -146,3 +146,18 @@ def test_lutgen32_matches_u8_expansion_and_extends_to_11(kind):
         i, j = np.meshgrid(np.arange(2048, dtype=np.uint32), np.arange(2048, dtype=np.uint32), indexing="ij")
         s = i + j
         assert np.array_equal(t, ((s >> 11) << 23) | ((s & 2047) << 12))
+
+
+def test_oracle_lut_product_against_reference_model_vectors(golden_dir):
+    """Golden vectors written by the reference's compiled models; pins the
+    oracle where oracle/_ref is not available (e.g. on the GPU box)."""
+    data = np.load(os.path.join(golden_dir, "product_vectors.npz"), allow_pickle=False)
+    for kind, m in LUT_FILES:
+        if kind == "ACC":
+            continue
+        a, b, want = data[f"{kind}_{m}_a"], data[f"{kind}_{m}_b"], data[f"{kind}_{m}_out"]
+        lut32 = cpu.expand_u8(lut_bytes(kind, m), m)
+        got = cpu.lut_mul_array(lut32, m, a.view(np.float32), b.view(np.float32))
+        assert same_bits_or_both_nan(got, want.view(np.float32)).all()
+        got = cpu.model_array(kind, m, a.view(np.float32), b.view(np.float32))
+        assert same_bits_or_both_nan(got, want.view(np.float32)).all()
