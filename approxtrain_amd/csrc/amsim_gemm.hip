@@ -9,13 +9,16 @@
 //     LUT gather all lanes share the uniform operand's mantissa, so the 64
 //     addresses fall into ONE 2^m-byte row of the byte-wide LUT image in LDS:
 //     at most 32 distinct dwords, one per bank -> no bank conflicts ever.
-//   * the uniform operand q is pre-decoded once per call into
-//     (sign|exponent as a power-of-two float, LUT row offset) pairs and read
-//     through the scalar cache (s_load), so it costs no VALU and no LDS.
-//   * the lane operand p is staged through LDS in [k][r] order by coalesced
-//     loads (dense, im2col-style patches, or filter-gradient gathers computed
-//     on the fly: no im2col / flipped-filter temporaries in HBM).
-//   * per MAC: v_add (LUT address), ds_read_u8, v_mul (2^ea * 2^eb),
+//   * the uniform operand q is pre-decoded once per call into one word per
+//     element (sign|exponent in the top 9 bits, LUT row offset in the low 16)
+//     laid out in 16-column tiles, and read through the scalar cache (s_load)
+//     four reduction rows at a time, so it costs no VALU and no LDS and the
+//     scalar-memory latency is paid once per 4 x TN MACs per lane.
+//   * the lane operand p is staged through LDS by coalesced (float4 where the
+//     source allows) loads -- dense, im2col-style patches, or filter-gradient
+//     gathers computed on the fly: no im2col / flipped-filter temporaries in
+//     HBM -- in a [k/4][r][4] layout that a lane reads back 16 bytes at a time.
+//   * per MAC: v_or (LUT address), ds_read_u8, v_mul (2^ea * 2^eb),
 //     v_lshl_add (byte -> 1.mant * 2^carry as a float), v_fma (accumulate).
 //     t * f is exact (power of two times an 8-bit significand), so the fused
 //     multiply-add rounds exactly like the reference's product-then-add.
@@ -32,14 +35,21 @@
 namespace amsim {
 
 constexpr int KC = 32;        // reduction depth of one staged chunk
+constexpr int KG = 4;         // reduction rows handled per scalar-load batch
+constexpr int NG = KC / KG;
+constexpr int QT = 16;        // columns per tile of the pre-decoded uniform operand
 constexpr int WG_THREADS = 256;
 constexpr int LUT_LDS_BYTES = 16384;
 constexpr int TARGET_WAVES = 4096;
 
 static std::atomic<int> g_split_k{1};
 
-typedef const __attribute__((address_space(4))) uint2 *cq2_t;
 typedef const __attribute__((address_space(4))) uint32_t *cq1_t;
+
+// staging modes of the lane operand
+enum { STAGE_R = 0,   // threads run along r, one element each (source contiguous in r)
+       STAGE_K = 1,   // threads run along k, one element each
+       STAGE_K4 = 2 };// threads run along k, four consecutive k per 16-byte load
 
 struct KArgs {
     PDesc p;
@@ -47,9 +57,9 @@ struct KArgs {
     int lut_bytes;
     int m;
     int lane_first;
-    const uint2 *qd;         // [qb][Kp][Jp] (t bits, row offset)
-    const uint32_t *qraw;    // [qb][Kp][Jp] raw bits
-    const uint32_t *qflags;  // [qb][nchunks]
+    const uint32_t *qw;      // [qb][Jp/16][Kp][16]  sign|exponent | row offset
+    const uint32_t *qraw;    // same layout, raw bits
+    const uint32_t *qflags;  // [qb][Jp/16][nchunks]
     int q_batches;
     int64_t R, J, K;
     int Jp, nchunks, nsplit, chunks_per_split;
@@ -67,23 +77,37 @@ struct QArgs {
     QDesc q;
     int64_t K, J;
     int Jp, nchunks, m;
-    uint2 *qd;
+    uint32_t *qw;
     uint32_t *qraw;
     uint32_t *qflags;
 };
 
+// One wavefront per (32-row chunk, 16-column tile): decodes the tile, writes it
+// in the tile-major layout the main kernel streams, and flags the tile-chunk
+// if it holds an operand the fast product path cannot take.
 __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
 {
-    const int ch = blockIdx.x, qb = blockIdx.y;
+    const int ch = blockIdx.x, qb = blockIdx.z;
+    const int lane = threadIdx.x & 63;
+    const int jt = blockIdx.y * (WG_THREADS / 64) + (threadIdx.x >> 6);
+    const int ntiles = a.Jp / QT;
+    if (jt >= ntiles) return;
     const float *base = a.q.base + (int64_t)qb * a.q.batch_stride;
-    const size_t plane = (size_t)a.nchunks * KC * a.Jp;
-    uint2 *qd = a.qd + (size_t)qb * plane + (size_t)ch * KC * a.Jp;
-    uint32_t *qraw = a.qraw + (size_t)qb * plane + (size_t)ch * KC * a.Jp;
+    const size_t Kp = (size_t)a.nchunks * KC;
+    const size_t tile = ((size_t)qb * ntiles + jt) * Kp * QT + (size_t)ch * KC * QT;
+    uint32_t *qw = a.qw + tile;
+    uint32_t *qraw = a.qraw + tile;
+    // lanes follow the source's contiguous direction
+    const bool k_fast = (a.q.kind == Q_DENSE && a.q.sk == 1 && a.q.sj != 1) || (a.q.kind == Q_FLIP);
     int unsafe = 0;
-    const int n = KC * a.Jp;
-    for (int e = threadIdx.x; e < n; e += WG_THREADS) {
-        const int kk = e / a.Jp, j = e - kk * a.Jp;
+#pragma unroll
+    for (int i = 0; i < KC * QT / 64; ++i) {
+        const int e = lane + 64 * i;
+        int kk, jj;
+        if (k_fast) { kk = e % KC; jj = e / KC; }
+        else { jj = e % QT; kk = e / QT; }
         const int64_t k = (int64_t)ch * KC + kk;
+        const int64_t j = (int64_t)jt * QT + jj;
         uint32_t raw = 0;
         if (k < a.K && j < a.J) {
             if (a.q.kind == Q_DENSE) {
@@ -97,67 +121,63 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
         }
         unsafe |= operand_unsafe(raw) ? 1 : 0;
         const uint32_t mant = (raw & 0x7fffffu) >> (23 - a.m);
-        qd[e] = make_uint2(raw & 0xff800000u, mant << a.m);
-        qraw[e] = raw;
+        qw[kk * QT + jj] = (raw & 0xff800000u) | (mant << a.m);
+        qraw[kk * QT + jj] = raw;
     }
-    unsafe = __syncthreads_or(unsafe);
-    if (threadIdx.x == 0) a.qflags[(size_t)qb * a.nchunks + ch] = (uint32_t)unsafe;
+    const int any = __any(unsafe);
+    if (lane == 0) a.qflags[((size_t)qb * ntiles + jt) * a.nchunks + ch] = (uint32_t)any;
 }
 
 // ---------------------------------------------------------------------------
-// lane-operand loaders
+// lane-operand row bookkeeping, kept in LDS: one int4 per local row.
+//   P_PATCH: {source offset of image b, y*sy - pt, x*sx - pl, 0}; rows past the
+//            end get a y origin far outside the source.
+//   P_GF:    {(fy*SW + fx)*C + c, fy, fx, 0}; rows past the end get fy far outside.
 // ---------------------------------------------------------------------------
-// Row bookkeeping kept in LDS: three ints per local row.
-//   P_PATCH: {source offset of image b, y*sy - pt, x*sx - pl}; invalid rows get
-//            a y origin far outside the source.
-//   P_GF:    {(fy*SW + fx)*C + c, fy, fx}; invalid rows get fy far outside.
-__device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t row0, int rows, int *ri)
+__device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t row0, int rows, int4 *ri)
 {
     for (int rl = threadIdx.x; rl < rows; rl += WG_THREADS) {
         const int64_t r = row0 + rl;
-        int a0 = 0, a1 = -(1 << 28), a2 = 0;
+        int4 v = make_int4(0, -(1 << 28), 0, 0);
         if (r < R) {
             if (p.kind == P_PATCH) {
                 const int x = (int)(r % p.GW);
                 const int64_t t = r / p.GW;
                 const int y = (int)(t % p.GH);
                 const int b = (int)(t / p.GH);
-                a0 = b * p.SH * p.SW * p.C;
-                a1 = y * p.sy - p.pt;
-                a2 = x * p.sx - p.pl;
+                v = make_int4(b * p.SH * p.SW * p.C, y * p.sy - p.pt, x * p.sx - p.pl, 0);
             } else if (p.kind == P_GF) {
                 const int c = (int)(r % p.C);
                 const int t = (int)(r / p.C);
                 const int fx = t % p.KW, fy = t / p.KW;
-                a0 = (fy * p.SW + fx) * p.C + c;
-                a1 = fy;
-                a2 = fx;
+                v = make_int4((fy * p.SW + fx) * p.C + c, fy, fx, 0);
             }
         }
-        ri[rl * 3 + 0] = a0;
-        ri[rl * 3 + 1] = a1;
-        ri[rl * 3 + 2] = a2;
+        ri[rl] = v;
     }
 }
+
+__device__ __forceinline__ int ch_begin_of(const KArgs &a, int split) { return split * a.chunks_per_split; }
 
 // ---------------------------------------------------------------------------
 // main kernel
 // ---------------------------------------------------------------------------
-// TN       outputs per lane (uniform-dimension tile of one wave)
-// WR       row tiles per workgroup (waves are arranged WR x 4/WR)
-// PK       lane-operand loader
-// ALONG_K  staging threads run along k (source contiguous in k) or along r
-template <int TN, int WR, int PK, bool ALONG_K>
+// TN     outputs per lane (uniform-dimension tile of one wave)
+// WR     row tiles per workgroup (waves are arranged WR x 4/WR)
+// PK     lane-operand source (PKind)
+// STAGE  how the staging threads walk the tile (STAGE_*)
+template <int TN, int WR, int PK, int STAGE>
 __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
 {
     constexpr int WC = 4 / WR;
     constexpr int ROWS = 64 * WR;
-    constexpr int RS = ROWS + (ALONG_K ? 1 : 0);  // padded row stride: conflict-free transposing stores
+    constexpr int GS = ROWS + 1;  // padded group stride (in uint4): conflict-free transposing stores
     constexpr int ELEMS = ROWS * KC / WG_THREADS;
+    constexpr int QUADS = ELEMS / 4;
 
     __shared__ __align__(16) uint8_t lut_s[LUT_LDS_BYTES];
-    __shared__ uint32_t Pt[KC * RS];
-    __shared__ int rowinfo[ROWS * 3];
+    __shared__ uint4 Pt4[NG * GS];
+    __shared__ int4 rowinfo[PK == P_DENSE ? 1 : ROWS];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -176,35 +196,106 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
 
     const float *pbase = a.p.base + (int64_t)bz * a.p.batch_stride;
     const int qb = a.q_batches > 1 ? bz : 0;
-    const size_t qplane = (size_t)a.nchunks * KC * a.Jp;
+    const size_t Kp = (size_t)a.nchunks * KC;
     // The pre-decoded uniform operand was written by an earlier kernel and is
     // read-only here: address it through the constant address space so that the
     // wave-uniform reads become scalar loads (s_load) into SGPRs.
-    const cq2_t qd = (cq2_t)(uintptr_t)(a.qd + (size_t)qb * qplane);
-    const cq1_t qraw = (cq1_t)(uintptr_t)(a.qraw + (size_t)qb * qplane);
-    const cq1_t qflags = (cq1_t)(uintptr_t)(a.qflags + (size_t)qb * a.nchunks);
+    const size_t qtile = ((size_t)qb * (a.Jp / QT) + (size_t)(j0 / QT)) * Kp * QT + (size_t)(j0 % QT);
+    const cq1_t qw = (cq1_t)(uintptr_t)(a.qw + qtile);
+    const cq1_t qraw = (cq1_t)(uintptr_t)(a.qraw + qtile);
+    const cq1_t qflags = (cq1_t)(uintptr_t)(a.qflags + ((size_t)qb * (a.Jp / QT) + (size_t)(j0 / QT)) * a.nchunks);
 
     const int ch_begin = split * a.chunks_per_split;
     const int ch_end = min(a.nchunks, ch_begin + a.chunks_per_split);
+
+    // Dense sources: one per-thread pointer to the first element this thread
+    // stages, a uniform step between its successive elements, and a uniform
+    // advance per chunk -- keeps the address arithmetic out of the scalar
+    // registers the inner loop needs for the uniform operand.
+    const float *dptr = nullptr;
+    int64_t dstep = 0, dchunk = 0;
+    int drow = 0, dvalid_rows = 0;
+    if (PK == P_DENSE) {
+        const int64_t left = a.R - row0;
+        dvalid_rows = (int)(left < ROWS ? left : ROWS);
+        if (STAGE == STAGE_K4) {
+            drow = tid >> 3;
+            dptr = pbase + (row0 + drow) * a.p.sr + (tid & (KC / 4 - 1)) * 4;
+            dstep = (int64_t)(WG_THREADS / (KC / 4)) * a.p.sr;
+            dchunk = KC;
+        } else if (STAGE == STAGE_K) {
+            drow = tid >> 5;
+            dptr = pbase + (row0 + drow) * a.p.sr + (int64_t)(tid & (KC - 1)) * a.p.sk;
+            dstep = (int64_t)(WG_THREADS / KC) * a.p.sr;
+            dchunk = (int64_t)KC * a.p.sk;
+        } else {
+            drow = tid & (ROWS - 1);
+            dptr = pbase + (row0 + drow) * a.p.sr + (int64_t)(tid / ROWS) * a.p.sk;
+            dstep = (int64_t)(WG_THREADS / ROWS) * a.p.sk;
+            dchunk = (int64_t)KC * a.p.sk;
+        }
+        // pin the walking state into vector registers
+        asm volatile("" : "+v"(dstep), "+v"(dchunk));
+        dptr += (int64_t)ch_begin_of(a, split) * dchunk;
+    }
 
     uint32_t pv[ELEMS];
     auto load_chunk = [&](int ch) -> int {
         const int64_t k0 = (int64_t)ch * KC;
         int unsafe = 0;
-        if (PK == P_DENSE) {
+        if (STAGE == STAGE_K4) {
+            // thread -> (row, quad of 4 consecutive k); all four share (fy, fx) because C % 4 == 0
+            const int kq = (tid & (KC / 4 - 1)) * 4;
+            const int64_t k = k0 + kq;
+            const bool kvalid = k < a.K;  // K % 4 == 0 on this path
+            int c = 0, fy = 0, fx = 0;
+            if (PK == P_PATCH) {
+                c = (int)(k % a.p.C);
+                const int t = (int)(k / a.p.C);
+                fx = t % a.p.KW; fy = t / a.p.KW;
+            }
+#pragma unroll
+            for (int i = 0; i < QUADS; ++i) {
+                const int rl = (tid >> 3) + i * (WG_THREADS / (KC / 4));
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (PK == P_DENSE) {
+                    // dptr walks this thread's first row; rows i*32 further down are dstep apart
+                    if (kvalid && drow + i * (WG_THREADS / (KC / 4)) < dvalid_rows)
+                        v = *reinterpret_cast<const uint4 *>(dptr + (int64_t)i * dstep);
+                } else {
+                    const int4 ri = rowinfo[rl];
+                    const int vy = ri.y + fy, vx = ri.z + fx;
+                    if (kvalid && (unsigned)vy < (unsigned)a.p.VH && (unsigned)vx < (unsigned)a.p.VW) {
+                        int sy_ = vy, sx_ = vx;
+                        bool on_grid = true;
+                        if (a.p.dy != 1 || a.p.dx != 1) {
+                            sy_ = vy / a.p.dy; sx_ = vx / a.p.dx;
+                            on_grid = (sy_ * a.p.dy == vy) && (sx_ * a.p.dx == vx);
+                        }
+                        if (on_grid)
+                            v = *reinterpret_cast<const uint4 *>(pbase + ri.x + (sy_ * a.p.SW + sx_) * a.p.C + c);
+                    }
+                }
+                pv[4 * i + 0] = v.x; pv[4 * i + 1] = v.y; pv[4 * i + 2] = v.z; pv[4 * i + 3] = v.w;
+                unsafe |= (operand_unsafe(v.x) | operand_unsafe(v.y) | operand_unsafe(v.z) | operand_unsafe(v.w)) ? 1 : 0;
+            }
+            if (PK == P_DENSE) dptr += dchunk;
+        } else if (PK == P_DENSE) {
 #pragma unroll
             for (int i = 0; i < ELEMS; ++i) {
-                int rl, kk;
-                if (ALONG_K) { kk = tid & (KC - 1); rl = (tid >> 5) + i * (WG_THREADS / KC); }
-                else { rl = tid & (ROWS - 1); kk = i * (WG_THREADS / ROWS) + (tid / ROWS); }
-                const int64_t r = row0 + rl, k = k0 + kk;
                 uint32_t v = 0;
-                if (r < a.R && k < a.K) v = f2u(pbase[r * a.p.sr + k * a.p.sk]);
+                if (STAGE == STAGE_K) {
+                    if (k0 + (tid & (KC - 1)) < a.K && drow + i * (WG_THREADS / KC) < dvalid_rows)
+                        v = f2u(dptr[(int64_t)i * dstep]);
+                } else {
+                    const int kk = i * (WG_THREADS / ROWS) + (tid / ROWS);
+                    if (k0 + kk < a.K && drow < dvalid_rows) v = f2u(dptr[(int64_t)i * dstep]);
+                }
                 pv[i] = v;
                 unsafe |= operand_unsafe(v) ? 1 : 0;
             }
-        } else if (PK == P_PATCH) {
-            // ALONG_K: this thread's k is fixed for the chunk
+            dptr += dchunk;
+        } else if (PK == P_PATCH) {  // STAGE_K: this thread's k is fixed for the chunk
             const int kk = tid & (KC - 1);
             const int64_t k = k0 + kk;
             const bool kvalid = k < a.K;
@@ -214,24 +305,24 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
 #pragma unroll
             for (int i = 0; i < ELEMS; ++i) {
                 const int rl = (tid >> 5) + i * (WG_THREADS / KC);
-                const int vy = rowinfo[rl * 3 + 1] + fy, vx = rowinfo[rl * 3 + 2] + fx;
+                const int4 ri = rowinfo[rl];
+                const int vy = ri.y + fy, vx = ri.z + fx;
                 uint32_t v = 0;
                 if (kvalid && (unsigned)vy < (unsigned)a.p.VH && (unsigned)vx < (unsigned)a.p.VW) {
                     int sy_ = vy, sx_ = vx;
                     bool on_grid = true;
                     if (a.p.dy != 1 || a.p.dx != 1) {
-                        sy_ = vy / a.p.dy;
-                        sx_ = vx / a.p.dx;
+                        sy_ = vy / a.p.dy; sx_ = vx / a.p.dx;
                         on_grid = (sy_ * a.p.dy == vy) && (sx_ * a.p.dx == vx);
                     }
-                    if (on_grid) v = f2u(pbase[rowinfo[rl * 3 + 0] + (sy_ * a.p.SW + sx_) * a.p.C + c]);
+                    if (on_grid) v = f2u(pbase[ri.x + (sy_ * a.p.SW + sx_) * a.p.C + c]);
                 }
                 pv[i] = v;
                 unsafe |= operand_unsafe(v) ? 1 : 0;
             }
         } else {  // P_GF, staged along r
             const int rl = tid & (ROWS - 1);
-            const int roff = rowinfo[rl * 3 + 0], fy = rowinfo[rl * 3 + 1], fx = rowinfo[rl * 3 + 2];
+            const int4 ri = rowinfo[rl];
 #pragma unroll
             for (int i = 0; i < ELEMS; ++i) {
                 const int kk = i * (WG_THREADS / ROWS) + __builtin_amdgcn_readfirstlane(tid / ROWS);
@@ -243,9 +334,9 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
                     const int y = (int)(t % a.p.GH);
                     const int b = (int)(t / a.p.GH);
                     const int iy0 = y * a.p.sy - a.p.pt, ix0 = x * a.p.sx - a.p.pl;
-                    const int iy = iy0 + fy, ix = ix0 + fx;
+                    const int iy = iy0 + ri.y, ix = ix0 + ri.z;
                     if ((unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
-                        v = f2u(pbase[((int64_t)(b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + roff]);
+                        v = f2u(pbase[((int64_t)(b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + ri.x]);
                 }
                 pv[i] = v;
                 unsafe |= operand_unsafe(v) ? 1 : 0;
@@ -254,12 +345,22 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
         return unsafe;
     };
     auto store_chunk = [&]() {
+        if (STAGE == STAGE_K4) {
+            const int g = tid & (KC / 4 - 1);
 #pragma unroll
-        for (int i = 0; i < ELEMS; ++i) {
-            int rl, kk;
-            if (ALONG_K) { kk = tid & (KC - 1); rl = (tid >> 5) + i * (WG_THREADS / KC); }
-            else { rl = tid & (ROWS - 1); kk = i * (WG_THREADS / ROWS) + (tid / ROWS); }
-            Pt[kk * RS + rl] = pv[i];
+            for (int i = 0; i < QUADS; ++i) {
+                const int rl = (tid >> 3) + i * (WG_THREADS / (KC / 4));
+                Pt4[g * GS + rl] = make_uint4(pv[4 * i], pv[4 * i + 1], pv[4 * i + 2], pv[4 * i + 3]);
+            }
+        } else {
+            uint32_t *Pt = reinterpret_cast<uint32_t *>(Pt4);
+#pragma unroll
+            for (int i = 0; i < ELEMS; ++i) {
+                int rl, kk;
+                if (STAGE == STAGE_K) { kk = tid & (KC - 1); rl = (tid >> 5) + i * (WG_THREADS / KC); }
+                else { rl = tid & (ROWS - 1); kk = i * (WG_THREADS / ROWS) + (tid / ROWS); }
+                Pt[((kk >> 2) * GS + rl) * 4 + (kk & 3)] = pv[i];
+            }
         }
     };
 
@@ -279,29 +380,42 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
         if (ch + 1 < ch_end) unsafe = load_chunk(ch + 1);  // in flight during the MACs below
         if (!active) continue;
         const uint32_t q_unsafe = qflags[ch];
-        const size_t qoff = (size_t)ch * KC * a.Jp + j0;
+        const size_t qoff = (size_t)ch * KC * QT;
         if (!(p_unsafe | q_unsafe)) {
-            cq2_t qrow = qd + qoff;
-#pragma unroll 4
-            for (int kk = 0; kk < KC; ++kk) {
-                const uint32_t raw = Pt[kk * RS + lrow];
-                const float ta = u2f(raw & 0xff800000u);
-                const uint32_t ia = (raw & 0x7fffffu) >> mshift;
-                uint32_t L[TN];
+            cq1_t qrow = qw + qoff;
+#pragma unroll 1
+            for (int g = 0; g < NG; ++g) {
+                uint32_t qv[KG][TN];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) L[j] = lut_s[qrow[j].y + ia];
+                for (int r = 0; r < KG; ++r)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const float t = u2f(qrow[j].x) * ta;
-                    const float f = u2f((L[j] << 16) + 0x3f800000u);
-                    acc[j] = __builtin_fmaf(t, f, acc[j]);
+                    for (int j = 0; j < TN; ++j) qv[r][j] = qrow[r * QT + j];
+                const uint4 p4 = Pt4[g * GS + lrow];
+                const uint32_t praw[KG] = {p4.x, p4.y, p4.z, p4.w};
+#pragma unroll
+                for (int r = 0; r < KG; ++r) {
+                    // keep each row's scalar unpacking next to its use: without the fence the
+                    // scheduler hoists all 128 s_and results to the loop top and spills them
+                    __builtin_amdgcn_sched_barrier(0);
+                    const float ta = u2f(praw[r] & 0xff800000u);
+                    const uint32_t ia = __builtin_amdgcn_ubfe(praw[r], (uint32_t)mshift, (uint32_t)m);
+                    uint32_t L[TN];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) L[j] = lut_s[(qv[r][j] & 0xffffu) | ia];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        const float t = u2f(qv[r][j] & 0xff800000u) * ta;
+                        const float f = u2f((L[j] << 16) + 0x3f800000u);
+                        acc[j] = __builtin_fmaf(t, f, acc[j]);
+                    }
                 }
-                qrow += a.Jp;
+                qrow += KG * QT;
             }
         } else {
             cq1_t qrow = qraw + qoff;
+            const uint32_t *Pt = reinterpret_cast<const uint32_t *>(Pt4);
             for (int kk = 0; kk < KC; ++kk) {
-                const uint32_t raw = Pt[kk * RS + lrow];
+                const uint32_t raw = Pt[((kk >> 2) * GS + lrow) * 4 + (kk & 3)];
                 const uint32_t ia = (raw & 0x7fffffu) >> mshift;
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
@@ -309,7 +423,7 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
                     const uint32_t e16 = (uint32_t)lut_s[(((qr & 0x7fffffu) >> mshift) << m) + ia] << 16;
                     acc[j] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
                 }
-                qrow += a.Jp;
+                qrow += QT;
             }
         }
     }
@@ -356,7 +470,7 @@ __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
 struct Plan {
     int TN, WR, Jp, nchunks, nsplit, chunks_per_split;
     int64_t Rp;
-    size_t off_qd, off_qraw, off_flags, off_partial, total;
+    size_t off_qw, off_qraw, off_flags, off_partial, total;
 };
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -367,7 +481,7 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
     pl.TN = J >= 9 ? 16 : J >= 5 ? 8 : J >= 3 ? 4 : (int)std::max<int64_t>(J, 1);
     const int64_t jchunks = (J + pl.TN - 1) / pl.TN;
     pl.WR = jchunks >= 2 ? 1 : 4;
-    pl.Jp = (int)((J + 15) / 16 * 16);
+    pl.Jp = (int)((J + QT - 1) / QT * QT);
     pl.nchunks = (int)((K + KC - 1) / KC);
     const int rows = 64 * pl.WR;
     pl.Rp = (R + rows - 1) / rows * rows;
@@ -382,9 +496,9 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
     if (pl.nchunks == 0) { pl.nsplit = 1; pl.chunks_per_split = 0; }
     const size_t plane = (size_t)pl.nchunks * KC * pl.Jp;
     size_t off = 0;
-    pl.off_qd = off;      off = align256(off + (size_t)q_batches * plane * sizeof(uint2));
+    pl.off_qw = off;      off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
     pl.off_qraw = off;    off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
-    pl.off_flags = off;   off = align256(off + (size_t)q_batches * std::max(pl.nchunks, 1) * sizeof(uint32_t));
+    pl.off_flags = off;   off = align256(off + (size_t)q_batches * (pl.Jp / QT) * std::max(pl.nchunks, 1) * sizeof(uint32_t));
     pl.off_partial = off;
     if (pl.nsplit > 1) off = align256(off + (size_t)pl.nsplit * batch * pl.Rp * pl.Jp * sizeof(float));
     pl.total = off;
@@ -397,17 +511,24 @@ size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
     return make_plan(R, J, K, batch, q_batches).total;
 }
 
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
 template <int TN, int WR>
 static void launch_variant(const KArgs &ka, dim3 grid, hipStream_t stream)
 {
-    const bool along_k = ka.p.kind == P_PATCH || (ka.p.kind == P_DENSE && ka.p.sk == 1 && ka.p.sr != 1);
-    if (ka.p.kind == P_DENSE) {
-        if (along_k) lutgemm_kernel<TN, WR, P_DENSE, true><<<grid, WG_THREADS, 0, stream>>>(ka);
-        else lutgemm_kernel<TN, WR, P_DENSE, false><<<grid, WG_THREADS, 0, stream>>>(ka);
-    } else if (ka.p.kind == P_PATCH) {
-        lutgemm_kernel<TN, WR, P_PATCH, true><<<grid, WG_THREADS, 0, stream>>>(ka);
+    const PDesc &p = ka.p;
+    if (p.kind == P_DENSE) {
+        const bool k_contig = p.sk == 1 && p.sr != 1;
+        const bool vec = k_contig && (p.sr % 4 == 0) && (ka.K % 4 == 0) && (p.batch_stride % 4 == 0) && aligned16(p.base);
+        if (vec) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K4><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else if (k_contig) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else lutgemm_kernel<TN, WR, P_DENSE, STAGE_R><<<grid, WG_THREADS, 0, stream>>>(ka);
+    } else if (p.kind == P_PATCH) {
+        const bool vec = (p.C % 4 == 0) && aligned16(p.base);
+        if (vec) lutgemm_kernel<TN, WR, P_PATCH, STAGE_K4><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else lutgemm_kernel<TN, WR, P_PATCH, STAGE_K><<<grid, WG_THREADS, 0, stream>>>(ka);
     } else {
-        lutgemm_kernel<TN, WR, P_GF, false><<<grid, WG_THREADS, 0, stream>>>(ka);
+        lutgemm_kernel<TN, WR, P_GF, STAGE_R><<<grid, WG_THREADS, 0, stream>>>(ka);
     }
 }
 
@@ -436,10 +557,11 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     QArgs qa{};
     qa.q = d.q;
     qa.K = d.K; qa.J = d.J; qa.Jp = pl.Jp; qa.nchunks = pl.nchunks; qa.m = lut.m;
-    qa.qd = reinterpret_cast<uint2 *>(ws + pl.off_qd);
+    qa.qw = reinterpret_cast<uint32_t *>(ws + pl.off_qw);
     qa.qraw = reinterpret_cast<uint32_t *>(ws + pl.off_qraw);
     qa.qflags = reinterpret_cast<uint32_t *>(ws + pl.off_flags);
-    q_prepass_kernel<<<dim3(pl.nchunks, d.q.batches), WG_THREADS, 0, stream>>>(qa);
+    if (d.q.batches > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
+    q_prepass_kernel<<<dim3(pl.nchunks, (pl.Jp / QT + 3) / 4, d.q.batches), WG_THREADS, 0, stream>>>(qa);
     AMSIM_HIP_CHECK(hipGetLastError());
 
     KArgs ka{};
@@ -448,7 +570,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.lut_bytes = (int)(((size_t)1 << (2 * lut.m)) + 15) / 16 * 16;
     ka.m = lut.m;
     ka.lane_first = d.lane_first ? 1 : 0;
-    ka.qd = qa.qd; ka.qraw = qa.qraw; ka.qflags = qa.qflags;
+    ka.qw = qa.qw; ka.qraw = qa.qraw; ka.qflags = qa.qflags;
     ka.q_batches = d.q.batches;
     ka.R = d.R; ka.J = d.J; ka.K = d.K;
     ka.Jp = pl.Jp; ka.nchunks = pl.nchunks; ka.nsplit = pl.nsplit; ka.chunks_per_split = pl.chunks_per_split;
