@@ -40,7 +40,11 @@ constexpr int NG = KC / KG;
 constexpr int QT = 16;        // columns per tile of the pre-decoded uniform operand
 constexpr int WG_THREADS = 256;
 constexpr int LUT_LDS_BYTES = 16384;
-constexpr int TARGET_WAVES = 4096;
+constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels are compiled for
+constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
+constexpr int DEVICE_CUS = 256;               // MI355X; only steers work splitting, never correctness
+constexpr int WG_SLOTS = DEVICE_CUS * WAVES_PER_SIMD;  // workgroups resident at once
+constexpr int TARGET_WAVES = WG_SLOTS * 4;
 
 static std::atomic<int> g_split_k{1};
 
@@ -65,8 +69,9 @@ struct KArgs {
     int Jp, nchunks, nsplit, chunks_per_split;
     float *out;
     int64_t so_r, so_j, out_batch_stride;
-    float *partial;          // [nsplit][batch][Rp][Jp] when nsplit > 1
+    float *partial;          // [nsplit][batch][Rp][Jp] when nsplit > 1 (rows relative to row_base)
     int64_t Rp;
+    int64_t row_base;        // first row this launch covers
     int batch;
 };
 
@@ -167,7 +172,7 @@ __device__ __forceinline__ int ch_begin_of(const KArgs &a, int split) { return s
 // PK     lane-operand source (PKind)
 // STAGE  how the staging threads walk the tile (STAGE_*)
 template <int TN, int WR, int PK, int STAGE>
-__global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
+__global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lutgemm_kernel(KArgs a)
 {
     constexpr int WC = 4 / WR;
     constexpr int ROWS = 64 * WR;
@@ -183,9 +188,24 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave / WC, wc = wave % WC;
-    const int bz = blockIdx.z / a.nsplit, split = blockIdx.z % a.nsplit;
-    const int64_t row0 = (int64_t)blockIdx.x * ROWS;
-    const int j0 = (blockIdx.y * WC + wc) * TN;
+    // Workgroups are handed to the 8 XCDs round-robin in launch order, and each
+    // XCD has its own L2.  Renumber so that each XCD works on a contiguous run
+    // of tiles (row tile fastest, then column group, then split / batch): the
+    // workgroups that share uniform-operand tiles and input rows then share an L2.
+    unsigned bx, by, bzz;
+    {
+        const unsigned X = gridDim.x, Y = gridDim.y, T = X * Y * gridDim.z;
+        const unsigned L = (blockIdx.z * Y + blockIdx.y) * X + blockIdx.x;
+        const unsigned xcd = L % NUM_XCD, idx = L / NUM_XCD;
+        const unsigned chunk = T / NUM_XCD, rem = T % NUM_XCD;
+        const unsigned V = xcd * chunk + (xcd < rem ? xcd : rem) + idx;
+        bx = V % X;
+        by = (V / X) % Y;
+        bzz = V / (X * Y);
+    }
+    const int bz = bzz / a.nsplit, split = bzz % a.nsplit;
+    const int64_t row0 = a.row_base + (int64_t)bx * ROWS;
+    const int j0 = (by * WC + wc) * TN;
     const bool active = j0 < a.J;
     const int m = a.m;
 
@@ -438,7 +458,7 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
                 if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = acc[j];
         }
     } else {
-        float *o = a.partial + (((size_t)split * a.batch + bz) * a.Rp + r) * a.Jp + j0;
+        float *o = a.partial + (((size_t)split * a.batch + bz) * a.Rp + (r - a.row_base)) * a.Jp + j0;
 #pragma unroll
         for (int j = 0; j < TN; ++j) o[j] = acc[j];
     }
@@ -448,8 +468,9 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_kernel(KArgs a)
 struct RArgs {
     const float *partial;
     float *out;
-    int64_t R, J, Rp, so_r, so_j, out_batch_stride;
+    int64_t R, J, Rp, so_r, so_j, out_batch_stride;  // R rows starting at row_base
     int Jp, nsplit, batch;
+    int64_t row_base;
 };
 
 __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
@@ -458,18 +479,33 @@ __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
     const int bz = blockIdx.y;
     if (idx >= a.R * a.J) return;
     const int64_t r = idx / a.J, j = idx - r * a.J;
-    float s = 0.0f;
-    for (int sp = 0; sp < a.nsplit; ++sp)
-        s += a.partial[(((size_t)sp * a.batch + bz) * a.Rp + r) * a.Jp + j];
-    a.out[(int64_t)bz * a.out_batch_stride + r * a.so_r + j * a.so_j] = s;
+    // eight interleaved chains keep eight loads in flight; the combination order is fixed
+    float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const size_t stride = (size_t)a.batch * a.Rp * a.Jp;
+    const float *src = a.partial + ((size_t)bz * a.Rp + r) * a.Jp + j;
+    int sp = 0;
+    for (; sp + 8 <= a.nsplit; sp += 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) c[u] += src[(size_t)(sp + u) * stride];
+    }
+    for (int u = 0; sp < a.nsplit; ++sp, ++u) c[u] += src[(size_t)sp * stride];
+    const float s = ((c[0] + c[1]) + (c[2] + c[3])) + ((c[4] + c[5]) + (c[6] + c[7]));
+    a.out[(int64_t)bz * a.out_batch_stride + (a.row_base + r) * a.so_r + j * a.so_j] = s;
 }
 
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
+// A call is one launch, or two when the workgroup count is a little more than a
+// whole number of machine-filling rounds: the rows of the last, mostly empty
+// round ("tail") are then launched separately with the reduction split across
+// enough workgroups to fill the machine again.
 struct Plan {
-    int TN, WR, Jp, nchunks, nsplit, chunks_per_split;
-    int64_t Rp;
+    int TN, WR, Jp, nchunks;
+    int nsplit, chunks_per_split;  // of the main launch
+    int64_t Rp;                    // padded rows of the launch that writes partials
+    int64_t rows_main;             // rows covered by the main launch (== R when there is no tail)
+    int tail_nsplit, tail_chunks_per_split;
     size_t off_qw, off_qraw, off_flags, off_partial, total;
 };
 
@@ -494,6 +530,25 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
     pl.chunks_per_split = (pl.nchunks + pl.nsplit - 1) / pl.nsplit;
     pl.nsplit = (pl.nchunks + pl.chunks_per_split - 1) / std::max(pl.chunks_per_split, 1);
     if (pl.nchunks == 0) { pl.nsplit = 1; pl.chunks_per_split = 0; }
+    pl.rows_main = R;
+    pl.tail_nsplit = 1;
+    pl.tail_chunks_per_split = pl.nchunks;
+    if (g_split_k.load() && pl.nsplit == 1 && pl.WR == 1 && pl.nchunks >= 4) {
+        const int64_t wgs_per_rowtile = ((jchunks + 3) / 4) * batch;
+        const int64_t rowtiles = pl.Rp / rows;
+        const int64_t wgs = rowtiles * wgs_per_rowtile;
+        const int64_t full_rounds = wgs / WG_SLOTS;
+        const int64_t main_tiles = full_rounds * WG_SLOTS / wgs_per_rowtile;
+        const int64_t tail_wgs = (rowtiles - main_tiles) * wgs_per_rowtile;
+        if (full_rounds >= 1 && tail_wgs > 0 && tail_wgs * 2 <= WG_SLOTS) {
+            int ts = (int)std::min<int64_t>(WG_SLOTS / tail_wgs, pl.nchunks / 2);
+            if (ts >= 2) {
+                pl.rows_main = main_tiles * rows;
+                pl.tail_chunks_per_split = (pl.nchunks + ts - 1) / ts;
+                pl.tail_nsplit = (pl.nchunks + pl.tail_chunks_per_split - 1) / pl.tail_chunks_per_split;
+            }
+        }
+    }
     const size_t plane = (size_t)pl.nchunks * KC * pl.Jp;
     size_t off = 0;
     pl.off_qw = off;      off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
@@ -501,6 +556,8 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
     pl.off_flags = off;   off = align256(off + (size_t)q_batches * (pl.Jp / QT) * std::max(pl.nchunks, 1) * sizeof(uint32_t));
     pl.off_partial = off;
     if (pl.nsplit > 1) off = align256(off + (size_t)pl.nsplit * batch * pl.Rp * pl.Jp * sizeof(float));
+    else if (pl.tail_nsplit > 1)
+        off = align256(off + (size_t)pl.tail_nsplit * batch * (pl.Rp - pl.rows_main) * pl.Jp * sizeof(float));
     pl.total = off;
     return pl;
 }
@@ -540,7 +597,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM path needs a byte LUT image (mantissa width <= 7)");
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
-        RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch};
+        RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0};
         dim3 grid((unsigned)((d.R * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
         splitk_reduce_kernel<<<grid, WG_THREADS, 0, stream>>>(ra);
         AMSIM_HIP_CHECK(hipGetLastError());
@@ -573,37 +630,49 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.qw = qa.qw; ka.qraw = qa.qraw; ka.qflags = qa.qflags;
     ka.q_batches = d.q.batches;
     ka.R = d.R; ka.J = d.J; ka.K = d.K;
-    ka.Jp = pl.Jp; ka.nchunks = pl.nchunks; ka.nsplit = pl.nsplit; ka.chunks_per_split = pl.chunks_per_split;
+    ka.Jp = pl.Jp; ka.nchunks = pl.nchunks;
     ka.out = d.out; ka.so_r = d.so_r; ka.so_j = d.so_j; ka.out_batch_stride = d.out_batch_stride;
     ka.partial = reinterpret_cast<float *>(ws + pl.off_partial);
-    ka.Rp = pl.Rp;
     ka.batch = d.batch;
 
     const int rows = 64 * pl.WR, wc = 4 / pl.WR;
     const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;
-    const int64_t gz = (int64_t)d.batch * pl.nsplit;
-    if (gz > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch x split-K exceeds the grid limit");
-    dim3 grid((unsigned)(pl.Rp / rows), (unsigned)((jchunks + wc - 1) / wc), (unsigned)gz);
-    if (grid.y > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "uniform dimension exceeds the grid limit");
-    switch (pl.TN) {
-    case 16:
-        if (pl.WR == 1) launch_variant<16, 1>(ka, grid, stream);
-        else launch_variant<16, 4>(ka, grid, stream);
-        break;
-    case 8: launch_variant<8, 4>(ka, grid, stream); break;
-    case 4: launch_variant<4, 4>(ka, grid, stream); break;
-    case 2: launch_variant<2, 4>(ka, grid, stream); break;
-    default: launch_variant<1, 4>(ka, grid, stream); break;
-    }
-    AMSIM_HIP_CHECK(hipGetLastError());
+    const unsigned gy = (unsigned)((jchunks + wc - 1) / wc);
+    if (gy > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "uniform dimension exceeds the grid limit");
 
-    if (pl.nsplit > 1) {
-        RArgs ra{ka.partial, d.out, d.R, d.J, pl.Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp, pl.nsplit, d.batch};
-        dim3 rgrid((unsigned)((d.R * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
-        splitk_reduce_kernel<<<rgrid, WG_THREADS, 0, stream>>>(ra);
+    auto launch = [&](int64_t row_base, int64_t row_end, int nsplit, int cps) -> int {
+        KArgs k = ka;
+        k.row_base = row_base;
+        k.nsplit = nsplit;
+        k.chunks_per_split = cps;
+        k.Rp = (row_end - row_base + rows - 1) / rows * rows;
+        const int64_t gz = (int64_t)d.batch * nsplit;
+        if (gz > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch x split-K exceeds the grid limit");
+        dim3 grid((unsigned)(k.Rp / rows), gy, (unsigned)gz);
+        switch (pl.TN) {
+        case 16:
+            if (pl.WR == 1) launch_variant<16, 1>(k, grid, stream);
+            else launch_variant<16, 4>(k, grid, stream);
+            break;
+        case 8: launch_variant<8, 4>(k, grid, stream); break;
+        case 4: launch_variant<4, 4>(k, grid, stream); break;
+        case 2: launch_variant<2, 4>(k, grid, stream); break;
+        default: launch_variant<1, 4>(k, grid, stream); break;
+        }
         AMSIM_HIP_CHECK(hipGetLastError());
-    }
-    return AMSIM_OK;
+        if (nsplit > 1) {
+            const int64_t nrows = std::min(row_end, d.R) - row_base;
+            RArgs ra{k.partial, d.out, nrows, d.J, k.Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp, nsplit, d.batch, row_base};
+            dim3 rgrid((unsigned)((nrows * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
+            splitk_reduce_kernel<<<rgrid, WG_THREADS, 0, stream>>>(ra);
+            AMSIM_HIP_CHECK(hipGetLastError());
+        }
+        return AMSIM_OK;
+    };
+    int rc = launch(0, pl.rows_main, pl.nsplit, pl.chunks_per_split);
+    if (rc != AMSIM_OK) return rc;
+    if (pl.rows_main < d.R) rc = launch(pl.rows_main, d.R, pl.tail_nsplit, pl.tail_chunks_per_split);
+    return rc;
 }
 
 // ---------------------------------------------------------------------------
