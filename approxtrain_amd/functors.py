@@ -43,8 +43,8 @@ def _lut(lut):
 
 def mul(lut, a, b):
     """Elementwise approximate product (test hook)."""
-    lut = _lut(lut)
     a, b = _dev(a, "a"), _dev(b, "b")
+    lut = _lut(lut)
     if a.shape != b.shape:
         raise ValueError("shape mismatch")
     out = torch.empty_like(a)
@@ -55,8 +55,8 @@ def mul(lut, a, b):
 def gemm(lut, A, B, trans_a=False, trans_b=False, swap_operands=False):
     """C = op(A) . op(B) for rank-2 A, B, or a strided batch for rank-3
     operands (a rank-2 operand is shared by every batch item)."""
-    lut = _lut(lut)
     A, B = _dev(A, "A"), _dev(B, "B")
+    lut = _lut(lut)
     if A.dim() not in (2, 3) or B.dim() not in (2, 3):
         raise ValueError("operands must be rank 2 or 3")
     batch = max(A.shape[0] if A.dim() == 3 else 1, B.shape[0] if B.dim() == 3 else 1)
@@ -83,8 +83,8 @@ def gemm(lut, A, B, trans_a=False, trans_b=False, swap_operands=False):
 
 def convam(lut, input, filter, strides=(1, 1), padding="SAME"):
     """ConvamFunctor: NHWC input, HWIO filter -> NHWC output."""
-    lut = _lut(lut)
     x, w = _dev(input, "input"), _dev(filter, "filter")
+    lut = _lut(lut)
     n, h, wd, c = x.shape
     kh, kw, c2, oc = w.shape
     if c != c2:
@@ -102,8 +102,8 @@ def convam(lut, input, filter, strides=(1, 1), padding="SAME"):
 
 def convam_input_grad(lut, input_sizes, filter, out_backprop, strides=(1, 1), padding="SAME"):
     """ConvamInputGradFunctor: gradient w.r.t. the NHWC input of shape input_sizes."""
-    lut = _lut(lut)
     w, dy = _dev(filter, "filter"), _dev(out_backprop, "out_backprop")
+    lut = _lut(lut)
     n, h, wd, c = [int(v) for v in input_sizes]
     kh, kw, c2, oc = w.shape
     oh, pt = conv_geometry(h, kh, strides[0], padding)
@@ -124,8 +124,8 @@ def convam_input_grad(lut, input_sizes, filter, out_backprop, strides=(1, 1), pa
 
 def convam_filter_grad(lut, input, filter_sizes, out_backprop, strides=(1, 1), padding="SAME"):
     """ConvamFilterGradFunctor: gradient w.r.t. the HWIO filter of shape filter_sizes."""
-    lut = _lut(lut)
     x, dy = _dev(input, "input"), _dev(out_backprop, "out_backprop")
+    lut = _lut(lut)
     n, h, wd, c = x.shape
     kh, kw, c2, oc = [int(v) for v in filter_sizes]
     oh, pt = conv_geometry(h, kh, strides[0], padding)
@@ -148,8 +148,8 @@ def _dense_dims(x, w):
 
 
 def denseam(lut, inputs, weights):
-    lut = _lut(lut)
     x, w = _dev(inputs, "inputs"), _dev(weights, "weights")
+    lut = _lut(lut)
     batch, units, width = _dense_dims(x, w)
     out = torch.empty((batch, units), dtype=torch.float32, device=x.device)
     lib = load_library()
@@ -161,8 +161,8 @@ def denseam(lut, inputs, weights):
 
 def denseam_grad(lut, grad, inputs, weights):
     """DenseamGrad op: returns (grad_input, grad_weights)."""
-    lut = _lut(lut)
     x, w, dy = _dev(inputs, "inputs"), _dev(weights, "weights"), _dev(grad, "grad")
+    lut = _lut(lut)
     batch, units, width = _dense_dims(x, w)
     if tuple(dy.shape) != (batch, units):
         raise ValueError("grad must be [batch, units]")
@@ -179,8 +179,8 @@ def denseam_grad(lut, grad, inputs, weights):
 
 def matmulam(lut, a, b):
     """LaunchMatMul: rank-2 / rank-3 operands with the reference's batch rules."""
-    lut = _lut(lut)
     a, b = _dev(a, "a"), _dev(b, "b")
+    lut = _lut(lut)
     if a.dim() not in (2, 3) or b.dim() not in (2, 3):
         raise ValueError("Input a and b should be 2 dimensional or 3 dimensional and compitable batch size")
     ba = a.shape[0] if a.dim() == 3 else 0

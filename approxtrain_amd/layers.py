@@ -1,0 +1,167 @@
+"""Layer mirrors of the reference's Keras layers, as ``torch.nn.Module``s:
+``AMConv2D`` (python/keras/layers/am_convolutional.py:400-558), ``denseam``
+(python/keras/layers/amdenselayer.py:47-256) and the attention layers of
+``ammha/multihead_attention.py``.  Bias add, activations, softmax, scaling and
+reshapes are plain torch ops, exactly as they are stock TF ops in the
+reference; every multiplication of activations by weights goes through the
+approximate-multiplier ops."""
+import math
+
+import torch
+from torch import nn
+
+from . import functors
+from .amnn_ops import amconvolution_v2
+from .math_ops import matmulam
+
+
+def _glorot_uniform_(t, fan_in, fan_out):
+    limit = math.sqrt(6.0 / (fan_in + fan_out))
+    with torch.no_grad():
+        return t.uniform_(-limit, limit)
+
+
+class AMConv2D(nn.Module):
+    """2-D convolution over NHWC input with an HWIO kernel through op ``Convam``.
+    Same constructor vocabulary as the Keras layer: ``filters, kernel_size,
+    strides, padding ('valid' | 'same'), activation, use_bias, mant_mul_lut``."""
+
+    def __init__(self, filters, kernel_size, strides=(1, 1), padding="valid", activation=None, use_bias=True,
+                 mant_mul_lut='', in_channels=None, dilation_rate=(1, 1)):
+        super().__init__()
+        if not mant_mul_lut:
+            raise ValueError("mant_mul_lut must name a LUT file")
+        ks = (kernel_size, kernel_size) if isinstance(kernel_size, int) else tuple(kernel_size)
+        st = (strides, strides) if isinstance(strides, int) else tuple(strides)
+        dr = (dilation_rate, dilation_rate) if isinstance(dilation_rate, int) else tuple(dilation_rate)
+        if any(d != 1 for d in dr):
+            raise ValueError("Dilation is not supported in current implementation")
+        if padding.lower() not in ("valid", "same"):
+            raise ValueError("padding must be 'valid' or 'same'")
+        self.filters, self.kernel_size, self.strides = int(filters), ks, st
+        self.padding = padding.upper()
+        self.activation, self.use_bias, self.mant_mul_lut = activation, use_bias, mant_mul_lut
+        self.kernel = None
+        self.bias = None
+        if in_channels is not None:
+            self.build(in_channels)
+
+    def build(self, in_channels, device=None):
+        kh, kw = self.kernel_size
+        k = torch.empty(kh, kw, in_channels, self.filters, device=device)
+        _glorot_uniform_(k, kh * kw * in_channels, kh * kw * self.filters)
+        self.kernel = nn.Parameter(k)
+        if self.use_bias:
+            self.bias = nn.Parameter(torch.zeros(self.filters, device=device))
+
+    def forward(self, inputs):
+        if self.kernel is None:
+            self.build(inputs.shape[-1], inputs.device)
+        out = amconvolution_v2(inputs, self.kernel, strides=list(self.strides), padding=self.padding,
+                               data_format="NHWC", mant_mul_lut=self.mant_mul_lut)
+        if self.use_bias:
+            out = out + self.bias
+        return self.activation(out) if self.activation is not None else out
+
+    def get_config(self):
+        return {"filters": self.filters, "kernel_size": self.kernel_size, "strides": self.strides,
+                "padding": self.padding.lower(), "use_bias": self.use_bias, "mant_mul_lut": self.mant_mul_lut}
+
+
+class _Denseam(torch.autograd.Function):
+    """op ``Denseam`` with gradient op ``DenseamGrad`` (denseam.cc:36-57, 177-184;
+    gradient registration amdenselayer.py:258-260)."""
+
+    @staticmethod
+    def forward(ctx, inputs, weights, mant_mul_lut):
+        ctx.save_for_backward(inputs, weights)
+        ctx.lut = mant_mul_lut
+        return functors.denseam(mant_mul_lut, inputs, weights)
+
+    @staticmethod
+    def backward(ctx, grad):
+        inputs, weights = ctx.saved_tensors
+        grad_input, grad_weights = functors.denseam_grad(ctx.lut, grad.contiguous(), inputs, weights)
+        return grad_input, grad_weights, None
+
+
+class denseam(nn.Module):
+    """Dense layer through op ``Denseam``: ``activation(inputs . kernel + bias)``.
+    Inputs of rank > 2 are flattened to [-1, width] and go through the same op
+    (the reference routes them to an exact ``tensordot``, amdenselayer.py:215,
+    which silently bypasses the approximate multiplier)."""
+
+    def __init__(self, units, activation=None, use_bias=True, mant_mul_lut='', input_dim=None):
+        super().__init__()
+        if not mant_mul_lut:
+            raise ValueError("mant_mul_lut must name a LUT file")
+        self.units, self.activation, self.use_bias, self.mant_mul_lut = int(units), activation, use_bias, mant_mul_lut
+        self.kernel = None
+        self.bias = None
+        if input_dim is not None:
+            self.build(input_dim)
+
+    def build(self, input_dim, device=None):
+        k = torch.empty(input_dim, self.units, device=device)
+        _glorot_uniform_(k, input_dim, self.units)
+        self.kernel = nn.Parameter(k)
+        if self.use_bias:
+            self.bias = nn.Parameter(torch.zeros(self.units, device=device))
+
+    def forward(self, inputs):
+        if self.kernel is None:
+            self.build(inputs.shape[-1], inputs.device)
+        lead = inputs.shape[:-1]
+        out = _Denseam.apply(inputs.reshape(-1, inputs.shape[-1]), self.kernel, self.mant_mul_lut)
+        out = out.reshape(tuple(lead) + (self.units,))
+        if self.use_bias:
+            out = out + self.bias
+        return self.activation(out) if self.activation is not None else out
+
+    def get_config(self):
+        return {"units": self.units, "use_bias": self.use_bias, "mant_mul_lut": self.mant_mul_lut}
+
+
+class DotProductAttention(nn.Module):
+    """Scaled dot-product attention with both matrix products through
+    ``matmulam`` (multihead_attention.py:9-30)."""
+
+    def __init__(self, lut_file):
+        super().__init__()
+        self.lut_file = lut_file
+
+    def forward(self, queries, keys, values, d_k, mask=None):
+        scores = matmulam(queries, keys, transpose_b=True, mant_mul_lut=self.lut_file) / math.sqrt(float(d_k))
+        if mask is not None:
+            scores = scores + -1e9 * mask
+        weights = torch.softmax(scores, dim=-1)
+        return matmulam(weights, values, mant_mul_lut=self.lut_file)
+
+
+class MultiHeadAttention(nn.Module):
+    """AMMHA (multihead_attention.py:33-89): four ``denseam`` projections around
+    ``DotProductAttention``."""
+
+    def __init__(self, lut_file, h, d_k, d_v, d_model, input_dim=None):
+        super().__init__()
+        self.attention = DotProductAttention(lut_file)
+        self.heads, self.d_k, self.d_v, self.d_model = h, d_k, d_v, d_model
+        self.W_q = denseam(d_k, mant_mul_lut=lut_file, input_dim=input_dim)
+        self.W_k = denseam(d_k, mant_mul_lut=lut_file, input_dim=input_dim)
+        self.W_v = denseam(d_v, mant_mul_lut=lut_file, input_dim=input_dim)
+        self.W_o = denseam(d_model, mant_mul_lut=lut_file, input_dim=d_v if input_dim is not None else None)
+
+    def reshape_tensor(self, x, heads, flag):
+        if flag:
+            x = x.reshape(x.shape[0], x.shape[1], heads, -1).permute(0, 2, 1, 3)
+        else:
+            x = x.permute(0, 2, 1, 3)
+            x = x.reshape(x.shape[0], x.shape[1], self.d_k)
+        return x.contiguous()
+
+    def forward(self, queries, keys, values, mask=None):
+        q = self.reshape_tensor(self.W_q(queries), self.heads, True)
+        k = self.reshape_tensor(self.W_k(keys), self.heads, True)
+        v = self.reshape_tensor(self.W_v(values), self.heads, True)
+        o = self.attention(q, k, v, self.d_k, mask)
+        return self.W_o(self.reshape_tensor(o, self.heads, False))

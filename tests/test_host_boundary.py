@@ -1,0 +1,128 @@
+"""CPU-only checks of the drop-in boundary and the host logic: the C-ABI
+library loads and exports every symbol include/amsim.h declares, the geometry
+helper matches TensorFlow's VALID/SAME closed form, status plumbing works, and
+the Python wrappers validate arguments like the reference's wrappers do.  No
+kernel is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+import approxtrain_amd
+from approxtrain_amd import _lib
+from tests.util import tf_same_pads
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "amsim.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(amsim_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = approxtrain_amd.load_library()
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), f"libamsim.so lacks {n}"
+    # and the Python binding table covers the same set
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_status_strings():
+    lib = approxtrain_amd.load_library()
+    assert lib.amsim_status_string(0) == b"ok"
+    assert b"workspace" in lib.amsim_status_string(5)
+
+
+@pytest.mark.parametrize("i,k,s", [(56, 3, 1), (28, 5, 1), (14, 5, 1), (5, 3, 2), (20, 5, 2), (4, 4, 1), (8, 1, 2),
+                                   (7, 3, 3), (32, 5, 2)])
+def test_conv_geometry_matches_tensorflow_closed_form(i, k, s):
+    o, p = _lib.conv_geometry(i, k, s, "SAME")
+    oo, pb, _ = tf_same_pads(i, k, s)
+    assert (o, p) == (oo, pb)
+    o, p = _lib.conv_geometry(i, k, s, "VALID")
+    assert (o, p) == (max((i - k + s) // s, 0), 0)
+
+
+def test_conv_geometry_rejects_bad_padding():
+    lib = approxtrain_amd.load_library()
+    o, p = C.c_int(), C.c_int()
+    assert lib.amsim_conv_geometry(8, 3, 1, 7, C.byref(o), C.byref(p)) == 1
+    assert b"padding" in lib.amsim_last_error()
+
+
+def test_lut_file_name_errors_do_not_exit(tmp_path):
+    """The reference exits the process on LUT problems (approx_mul_lut.h:18-40);
+    the library returns a status."""
+    lib = approxtrain_amd.load_library()
+    h = C.c_void_p()
+    assert lib.amsim_lut_load_file(b"", C.byref(h)) == 1
+    assert lib.amsim_lut_load_file(b"/nonexistent/MBM_7.bin", C.byref(h)) == 2          # I/O
+    assert lib.amsim_lut_load_file(b"/nonexistent/nosuffix.bin", C.byref(h)) == 3       # no _<m>
+    assert lib.amsim_lut_load_file(b"/nonexistent/MBM_x7.bin", C.byref(h)) == 3        # width not a number
+    assert lib.amsim_lut_load_file(b"/nonexistent/MBM_9.bin", C.byref(h)) == 3         # byte LUTs stop at m = 7
+    short = tmp_path / "MBM_7.bin"
+    short.write_bytes(b"\x00" * 100)
+    assert lib.amsim_lut_load_file(str(short).encode(), C.byref(h)) == 3               # short file
+    assert not h.value
+
+
+def test_workspace_queries_need_no_device():
+    lib = approxtrain_amd.load_library()
+    assert lib.amsim_gemm_workspace_bytes(0, 0, 4096, 4096, 4096, 1) > 0
+    assert lib.amsim_convam_workspace_bytes(32, 56, 56, 64, 3, 3, 64) > 0
+    assert lib.amsim_convam_filter_grad_workspace_bytes(32, 56, 56, 64, 3, 3, 64) > 0
+    assert lib.amsim_gemm_workspace_bytes(0, 0, 0, 5, 5, 1) == 0
+    assert lib.amsim_matmulam_workspace_bytes(2, 3, 4, 5, 5, 6) == 0  # incompatible batches
+
+
+def test_functors_refuse_host_tensors():
+    from approxtrain_amd import functors
+    with pytest.raises(TypeError, match="device memory"):
+        functors.gemm("x_7.bin", torch.zeros(2, 2), torch.zeros(2, 2))
+
+
+def test_amconvolution_argument_validation():
+    from approxtrain_amd.amnn_ops import _get_sequence, amconvolution_v2
+    x, w = torch.zeros(1, 4, 4, 2), torch.zeros(3, 3, 2, 5)
+    assert _get_sequence(2, 2, 3, "strides") == [1, 2, 2, 1]
+    assert _get_sequence([2, 3], 2, 3, "strides") == [1, 2, 3, 1]
+    assert _get_sequence(None, 2, 3, "strides") == [1, 1, 1, 1]
+    with pytest.raises(ValueError):
+        _get_sequence([1, 2, 3], 2, 3, "strides")
+    with pytest.raises(ValueError, match="Dilation is not supported"):
+        amconvolution_v2(x, w, dilations=[1, 2, 2, 1], mant_mul_lut="MBM_7.bin")
+    with pytest.raises(ValueError, match="mant_mul_lut"):
+        amconvolution_v2(x, w)
+    with pytest.raises(ValueError, match="depth"):
+        amconvolution_v2(x, torch.zeros(3, 3, 3, 5), mant_mul_lut="MBM_7.bin")
+    with pytest.raises(ValueError):
+        amconvolution_v2(x, w, data_format="NCHW", mant_mul_lut="MBM_7.bin")
+
+
+def test_matmulam_argument_validation():
+    from approxtrain_amd.math_ops import matmulam
+    a, b = torch.zeros(2, 3), torch.zeros(3, 4)
+    with pytest.raises(ValueError, match="unsupported args"):
+        matmulam(a, b, adjoint_a=True, mant_mul_lut="MBM_7.bin")
+    with pytest.raises(ValueError, match="mant_mul_lut"):
+        matmulam(a, b)
+
+
+def test_layers_validate_constructor_arguments():
+    from approxtrain_amd.layers import AMConv2D, denseam
+    with pytest.raises(ValueError):
+        AMConv2D(8, 3, mant_mul_lut="")
+    with pytest.raises(ValueError, match="Dilation"):
+        AMConv2D(8, 3, dilation_rate=2, mant_mul_lut="MBM_7.bin")
+    with pytest.raises(ValueError):
+        denseam(8)
+    layer = AMConv2D(6, 5, padding="same", mant_mul_lut="MBM_7.bin", in_channels=1)
+    assert tuple(layer.kernel.shape) == (5, 5, 1, 6) and layer.get_config()["mant_mul_lut"] == "MBM_7.bin"
+    d = denseam(300, mant_mul_lut="MBM_7.bin", input_dim=784)
+    assert tuple(d.kernel.shape) == (784, 300)
