@@ -172,7 +172,8 @@ __device__ __forceinline__ int ch_begin_of(const KArgs &a, int split) { return s
 // PK     lane-operand source (PKind)
 // STAGE  how the staging threads walk the tile (STAGE_*)
 template <int TN, int WR, int PK, int STAGE>
-__global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lutgemm_kernel(KArgs a)
+__global__ __launch_bounds__(WG_THREADS, (WR != 1 ? 2 : (PK == P_DENSE && STAGE != STAGE_K4) ? WAVES_PER_SIMD - 1 : WAVES_PER_SIMD))
+void lutgemm_kernel(KArgs a)
 {
     constexpr int WC = 4 / WR;
     constexpr int ROWS = 64 * WR;
@@ -250,14 +251,42 @@ __global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lu
             dchunk = (int64_t)KC * a.p.sk;
         } else {
             drow = tid & (ROWS - 1);
-            dptr = pbase + (row0 + drow) * a.p.sr + (int64_t)(tid / ROWS) * a.p.sk;
-            dstep = (int64_t)(WG_THREADS / ROWS) * a.p.sk;
+            dptr = pbase + (row0 + drow) * a.p.sr + (int64_t)((tid / ROWS) * ELEMS) * a.p.sk;
+            dstep = a.p.sk;
             dchunk = (int64_t)KC * a.p.sk;
         }
         // pin the walking state into vector registers
         asm volatile("" : "+v"(dstep), "+v"(dchunk));
         dptr += (int64_t)ch_begin_of(a, split) * dchunk;
     }
+
+    // Patch sources: (fy, fx, c) of the first k of the next chunk to stage, walked
+    // chunk by chunk with scalar adds instead of being re-derived by division.
+    int cb_c = 0, cb_fx = 0, cb_fy = 0;
+    const bool patch_walk = PK == P_PATCH && a.p.C >= KC;
+    if (patch_walk) {
+        const int64_t kb = (int64_t)ch_begin_of(a, split) * KC;
+        cb_c = (int)(kb % a.p.C);
+        const int t = (int)(kb / a.p.C);
+        cb_fx = t % a.p.KW;
+        cb_fy = t / a.p.KW;
+    }
+    auto decompose_k = [&](int64_t k, int koff, int &c, int &fx, int &fy) {
+        if (patch_walk) {  // C >= KC: at most one wrap within a chunk
+            c = cb_c + koff; fx = cb_fx; fy = cb_fy;
+            if (c >= a.p.C) { c -= a.p.C; if (++fx == a.p.KW) { fx = 0; ++fy; } }
+        } else {
+            c = (int)(k % a.p.C);
+            const int t = (int)(k / a.p.C);
+            fx = t % a.p.KW; fy = t / a.p.KW;
+        }
+    };
+    auto advance_chunk_base = [&]() {
+        if (patch_walk) {
+            cb_c += KC;
+            if (cb_c >= a.p.C) { cb_c -= a.p.C; if (++cb_fx == a.p.KW) { cb_fx = 0; ++cb_fy; } }
+        }
+    };
 
     uint32_t pv[ELEMS];
     auto load_chunk = [&](int ch) -> int {
@@ -269,11 +298,7 @@ __global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lu
             const int64_t k = k0 + kq;
             const bool kvalid = k < a.K;  // K % 4 == 0 on this path
             int c = 0, fy = 0, fx = 0;
-            if (PK == P_PATCH) {
-                c = (int)(k % a.p.C);
-                const int t = (int)(k / a.p.C);
-                fx = t % a.p.KW; fy = t / a.p.KW;
-            }
+            if (PK == P_PATCH) decompose_k(k, kq, c, fx, fy);
 #pragma unroll
             for (int i = 0; i < QUADS; ++i) {
                 const int rl = (tid >> 3) + i * (WG_THREADS / (KC / 4));
@@ -308,7 +333,7 @@ __global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lu
                     if (k0 + (tid & (KC - 1)) < a.K && drow + i * (WG_THREADS / KC) < dvalid_rows)
                         v = f2u(dptr[(int64_t)i * dstep]);
                 } else {
-                    const int kk = i * (WG_THREADS / ROWS) + (tid / ROWS);
+                    const int kk = (tid / ROWS) * ELEMS + i;
                     if (k0 + kk < a.K && drow < dvalid_rows) v = f2u(dptr[(int64_t)i * dstep]);
                 }
                 pv[i] = v;
@@ -319,9 +344,8 @@ __global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lu
             const int kk = tid & (KC - 1);
             const int64_t k = k0 + kk;
             const bool kvalid = k < a.K;
-            const int c = (int)(k % a.p.C);
-            const int t = (int)(k / a.p.C);
-            const int fx = t % a.p.KW, fy = t / a.p.KW;
+            int c, fx, fy;
+            decompose_k(k, kk, c, fx, fy);
 #pragma unroll
             for (int i = 0; i < ELEMS; ++i) {
                 const int rl = (tid >> 5) + i * (WG_THREADS / KC);
@@ -340,28 +364,30 @@ __global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lu
                 pv[i] = v;
                 unsafe |= operand_unsafe(v) ? 1 : 0;
             }
-        } else {  // P_GF, staged along r
+        } else {  // P_GF, staged along r: this thread stages ELEMS consecutive k (pixels) of its row
             const int rl = tid & (ROWS - 1);
             const int4 ri = rowinfo[rl];
+            // the first pixel of this wave's run, decomposed once (wave-uniform), then walked
+            const int64_t kfirst = k0 + __builtin_amdgcn_readfirstlane(tid / ROWS) * ELEMS;
+            int x = (int)(kfirst % a.p.GW);
+            const int64_t t = kfirst / a.p.GW;
+            int y = (int)(t % a.p.GH);
+            int b = (int)(t / a.p.GH);
 #pragma unroll
             for (int i = 0; i < ELEMS; ++i) {
-                const int kk = i * (WG_THREADS / ROWS) + __builtin_amdgcn_readfirstlane(tid / ROWS);
-                const int64_t k = k0 + kk;
                 uint32_t v = 0;
-                if (k < a.K) {
-                    const int x = (int)(k % a.p.GW);
-                    const int64_t t = k / a.p.GW;
-                    const int y = (int)(t % a.p.GH);
-                    const int b = (int)(t / a.p.GH);
+                if (kfirst + i < a.K) {
                     const int iy0 = y * a.p.sy - a.p.pt, ix0 = x * a.p.sx - a.p.pl;
                     const int iy = iy0 + ri.y, ix = ix0 + ri.z;
                     if ((unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
-                        v = f2u(pbase[((int64_t)(b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + ri.x]);
+                        v = f2u(pbase[((b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + ri.x]);
                 }
                 pv[i] = v;
                 unsafe |= operand_unsafe(v) ? 1 : 0;
+                if (++x == a.p.GW) { x = 0; if (++y == a.p.GH) { y = 0; ++b; } }
             }
         }
+        if (PK == P_PATCH) advance_chunk_base();
         return unsafe;
     };
     auto store_chunk = [&]() {
@@ -372,13 +398,19 @@ __global__ __launch_bounds__(WG_THREADS, (WR == 1 ? WAVES_PER_SIMD : 2)) void lu
                 const int rl = (tid >> 3) + i * (WG_THREADS / (KC / 4));
                 Pt4[g * GS + rl] = make_uint4(pv[4 * i], pv[4 * i + 1], pv[4 * i + 2], pv[4 * i + 3]);
             }
+        } else if (STAGE == STAGE_R) {
+            // ELEMS consecutive k of row rl, starting at a multiple of 4: whole uint4 groups
+            const int rl = tid & (ROWS - 1);
+            const int g0 = (tid / ROWS) * (ELEMS / 4);
+#pragma unroll
+            for (int i = 0; i < ELEMS / 4; ++i)
+                Pt4[(g0 + i) * GS + rl] = make_uint4(pv[4 * i], pv[4 * i + 1], pv[4 * i + 2], pv[4 * i + 3]);
         } else {
             uint32_t *Pt = reinterpret_cast<uint32_t *>(Pt4);
+            const int kk = tid & (KC - 1);
 #pragma unroll
             for (int i = 0; i < ELEMS; ++i) {
-                int rl, kk;
-                if (STAGE == STAGE_K) { kk = tid & (KC - 1); rl = (tid >> 5) + i * (WG_THREADS / KC); }
-                else { rl = tid & (ROWS - 1); kk = i * (WG_THREADS / ROWS) + (tid / ROWS); }
+                const int rl = (tid >> 5) + i * (WG_THREADS / KC);
                 Pt[((kk >> 2) * GS + rl) * 4 + (kk & 3)] = pv[i];
             }
         }

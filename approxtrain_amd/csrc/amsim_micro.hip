@@ -85,11 +85,32 @@ __global__ __launch_bounds__(MICRO_THREADS) void micro_lds_kernel(int iters, flo
     if (acc == 0x12345u) sink[threadIdx.x] = (float)acc;
 }
 
+// plain streaming copy: the known-size kernel that hardware traffic counters are scaled against
+__global__ __launch_bounds__(MICRO_THREADS) void calibration_copy_kernel(const float4 *src, float4 *dst, size_t n4)
+{
+    size_t i = (size_t)blockIdx.x * MICRO_THREADS + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * MICRO_THREADS;
+    for (; i < n4; i += stride) dst[i] = src[i];
+}
+
 }  // namespace amsim
 
 using namespace amsim;
 
 extern "C" {
+
+// Copies n floats (n a multiple of 4, 16-byte aligned buffers) with a plain
+// kernel: reads 4n bytes, writes 4n bytes.
+int amsim_calibration_copy(const float *src, float *dst, size_t n, void *stream)
+{
+    if (!src || !dst || (n & 3) || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15))
+        return fail(AMSIM_ERR_INVALID, "calibration copy needs 16-byte aligned buffers and n % 4 == 0");
+    if (n == 0) return AMSIM_OK;
+    calibration_copy_kernel<<<2048, MICRO_THREADS, 0, static_cast<hipStream_t>(stream)>>>(
+        reinterpret_cast<const float4 *>(src), reinterpret_cast<float4 *>(dst), n / 4);
+    AMSIM_HIP_CHECK(hipGetLastError());
+    return AMSIM_OK;
+}
 
 // Runs micro-kernel `kind` (0 = VALU FMA, 1..6 = LDS gather modes 0..5,
 // 10..14 = VALU modes 0..4 with `sink[512..]` receiving the shader-clock ticks

@@ -143,6 +143,14 @@ def main():
         torch.cuda.synchronize()
         pass_ms[name] = e0.elapsed_time(e1) / args.steps
 
+    # one plain copy of known size (64 MiB read + 64 MiB written), outside every timed
+    # region: the kernel that FETCH_SIZE / WRITE_SIZE counter readings are scaled against
+    cal_src = torch.ones(16 * 1024 * 1024, device="cuda")
+    cal_dst = torch.empty_like(cal_src)
+    lib.amsim_calibration_copy(C.c_void_p(cal_src.data_ptr()), C.c_void_p(cal_dst.data_ptr()), cal_src.numel(),
+                               C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+
     peaks = measure_peaks(lib, cus.value)
     valu_bound = peaks["valu_mix_lane_ops_per_s"] / VALU_OPS_PER_MAC / 1e9
     lds_bound = peaks["lds_u8_row_gathers_per_s"] / 1e9

@@ -161,6 +161,11 @@ int amsim_set_split_k(int mode);
 int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream, float *sink,
                      double *ms_per_launch, double *ops_per_launch);
 
+/* Plain copy kernel of known size (reads 4n bytes, writes 4n bytes; n % 4 == 0,
+ * 16-byte aligned buffers): the reference point that hardware traffic counters
+ * (FETCH_SIZE / WRITE_SIZE) are scaled against. */
+int amsim_calibration_copy(const float *src, float *dst, size_t n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
