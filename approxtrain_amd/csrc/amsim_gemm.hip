@@ -57,7 +57,7 @@ enum { STAGE_R = 0,   // threads run along r, one element each (source contiguou
 
 struct KArgs {
     PDesc p;
-    const uint8_t *lut_img;  // byte image: (uniform mantissa << m) | lane mantissa
+    const uint8_t *lut_img;  // LUT image indexed (uniform mantissa << m) | lane mantissa: bytes, or uint16 for m > 7
     int lut_bytes;
     int m;
     int lane_first;
@@ -171,7 +171,10 @@ __device__ __forceinline__ int ch_begin_of(const KArgs &a, int split) { return s
 // WR     row tiles per workgroup (waves are arranged WR x 4/WR)
 // PK     lane-operand source (PKind)
 // STAGE  how the staging threads walk the tile (STAGE_*)
-template <int TN, int WR, int PK, int STAGE>
+// LUTG   false: byte LUT image resident in LDS (mantissa width <= 7)
+//        true:  16-bit LUT image gathered from global memory through L2 / MALL
+//               (widths 8..11; a 2^22-entry table does not fit the 160 KB LDS)
+template <int TN, int WR, int PK, int STAGE, bool LUTG>
 __global__ __launch_bounds__(WG_THREADS, (WR != 1 ? 2 : (PK == P_DENSE && STAGE != STAGE_K4) ? WAVES_PER_SIMD - 1 : WAVES_PER_SIMD))
 void lutgemm_kernel(KArgs a)
 {
@@ -181,7 +184,9 @@ void lutgemm_kernel(KArgs a)
     constexpr int ELEMS = ROWS * KC / WG_THREADS;
     constexpr int QUADS = ELEMS / 4;
 
-    __shared__ __align__(16) uint8_t lut_s[LUT_LDS_BYTES];
+    __shared__ __align__(16) uint8_t lut_s[LUTG ? 16 : LUT_LDS_BYTES];
+    const uint16_t *__restrict__ lut_g = reinterpret_cast<const uint16_t *>(a.lut_img);
+    constexpr int ESHIFT = LUTG ? 8 : 16;  // LUT entry -> carry << 23 | mantissa
     __shared__ uint4 Pt4[NG * GS];
     __shared__ int4 rowinfo[PK == P_DENSE ? 1 : ROWS];
 
@@ -210,8 +215,9 @@ void lutgemm_kernel(KArgs a)
     const bool active = j0 < a.J;
     const int m = a.m;
 
-    for (int i = tid * 16; i < a.lut_bytes; i += WG_THREADS * 16)
-        *reinterpret_cast<uint4 *>(lut_s + i) = *reinterpret_cast<const uint4 *>(a.lut_img + i);
+    if (!LUTG)
+        for (int i = tid * 16; i < a.lut_bytes; i += WG_THREADS * 16)
+            *reinterpret_cast<uint4 *>(lut_s + i) = *reinterpret_cast<const uint4 *>(a.lut_img + i);
     if (PK != P_DENSE) fill_rowinfo(a.p, a.R, row0, ROWS, rowinfo);
     __syncthreads();
 
@@ -453,11 +459,14 @@ void lutgemm_kernel(KArgs a)
                     const uint32_t ia = __builtin_amdgcn_ubfe(praw[r], (uint32_t)mshift, (uint32_t)m);
                     uint32_t L[TN];
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) L[j] = lut_s[(qv[r][j] & 0xffffu) | ia];
+                    for (int j = 0; j < TN; ++j) {
+                        const uint32_t li = (qv[r][j] & 0x7fffffu) | ia;
+                        L[j] = LUTG ? (uint32_t)lut_g[li] : (uint32_t)lut_s[li];
+                    }
 #pragma unroll
                     for (int j = 0; j < TN; ++j) {
                         const float t = u2f(qv[r][j] & 0xff800000u) * ta;
-                        const float f = u2f((L[j] << 16) + 0x3f800000u);
+                        const float f = u2f((L[j] << ESHIFT) + 0x3f800000u);
                         acc[j] = __builtin_fmaf(t, f, acc[j]);
                     }
                 }
@@ -472,7 +481,8 @@ void lutgemm_kernel(KArgs a)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     const uint32_t qr = qrow[j];
-                    const uint32_t e16 = (uint32_t)lut_s[(((qr & 0x7fffffu) >> mshift) << m) + ia] << 16;
+                    const uint32_t li = (((qr & 0x7fffffu) >> mshift) << m) + ia;
+                    const uint32_t e16 = (LUTG ? (uint32_t)lut_g[li] : (uint32_t)lut_s[li]) << ESHIFT;
                     acc[j] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
                 }
                 qrow += QT;
@@ -602,22 +612,37 @@ size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-template <int TN, int WR>
+template <int TN, int WR, bool LUTG>
 static void launch_variant(const KArgs &ka, dim3 grid, hipStream_t stream)
 {
     const PDesc &p = ka.p;
     if (p.kind == P_DENSE) {
         const bool k_contig = p.sk == 1 && p.sr != 1;
         const bool vec = k_contig && (p.sr % 4 == 0) && (ka.K % 4 == 0) && (p.batch_stride % 4 == 0) && aligned16(p.base);
-        if (vec) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K4><<<grid, WG_THREADS, 0, stream>>>(ka);
-        else if (k_contig) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K><<<grid, WG_THREADS, 0, stream>>>(ka);
-        else lutgemm_kernel<TN, WR, P_DENSE, STAGE_R><<<grid, WG_THREADS, 0, stream>>>(ka);
+        if (vec) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K4, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else if (k_contig) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else lutgemm_kernel<TN, WR, P_DENSE, STAGE_R, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
     } else if (p.kind == P_PATCH) {
         const bool vec = (p.C % 4 == 0) && aligned16(p.base);
-        if (vec) lutgemm_kernel<TN, WR, P_PATCH, STAGE_K4><<<grid, WG_THREADS, 0, stream>>>(ka);
-        else lutgemm_kernel<TN, WR, P_PATCH, STAGE_K><<<grid, WG_THREADS, 0, stream>>>(ka);
+        if (vec) lutgemm_kernel<TN, WR, P_PATCH, STAGE_K4, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else lutgemm_kernel<TN, WR, P_PATCH, STAGE_K, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
     } else {
-        lutgemm_kernel<TN, WR, P_GF, STAGE_R><<<grid, WG_THREADS, 0, stream>>>(ka);
+        lutgemm_kernel<TN, WR, P_GF, STAGE_R, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
+    }
+}
+
+template <bool LUTG>
+static void launch_tn(int TN, int WR, const KArgs &k, dim3 grid, hipStream_t stream)
+{
+    switch (TN) {
+    case 16:
+        if (WR == 1) launch_variant<16, 1, LUTG>(k, grid, stream);
+        else launch_variant<16, 4, LUTG>(k, grid, stream);
+        break;
+    case 8: launch_variant<8, 4, LUTG>(k, grid, stream); break;
+    case 4: launch_variant<4, 4, LUTG>(k, grid, stream); break;
+    case 2: launch_variant<2, 4, LUTG>(k, grid, stream); break;
+    default: launch_variant<1, 4, LUTG>(k, grid, stream); break;
     }
 }
 
@@ -625,8 +650,8 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
 {
     if (d.R < 0 || d.J < 0 || d.K < 0 || d.batch < 0) return fail(AMSIM_ERR_INVALID, "negative GEMM extent");
     if (d.R == 0 || d.J == 0 || d.batch == 0) return AMSIM_OK;
-    if (lut.m > 7 || lut.img_ab == nullptr)
-        return fail(AMSIM_ERR_UNSUPPORTED, "GEMM path needs a byte LUT image (mantissa width <= 7)");
+    if ((lut.m <= 7 && lut.img_ab == nullptr) || (lut.m > 7 && lut.img16_ab == nullptr))
+        return fail(AMSIM_ERR_UNSUPPORTED, "LUT handle holds no device image for the GEMM path");
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
         RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0};
@@ -655,7 +680,8 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
 
     KArgs ka{};
     ka.p = d.p;
-    ka.lut_img = d.lane_first ? lut.img_ba : lut.img_ab;
+    if (lut.m <= 7) ka.lut_img = d.lane_first ? lut.img_ba : lut.img_ab;
+    else ka.lut_img = reinterpret_cast<const uint8_t *>(d.lane_first ? lut.img16_ba : lut.img16_ab);
     ka.lut_bytes = (int)(((size_t)1 << (2 * lut.m)) + 15) / 16 * 16;
     ka.m = lut.m;
     ka.lane_first = d.lane_first ? 1 : 0;
@@ -681,16 +707,8 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         const int64_t gz = (int64_t)d.batch * nsplit;
         if (gz > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch x split-K exceeds the grid limit");
         dim3 grid((unsigned)(k.Rp / rows), gy, (unsigned)gz);
-        switch (pl.TN) {
-        case 16:
-            if (pl.WR == 1) launch_variant<16, 1>(k, grid, stream);
-            else launch_variant<16, 4>(k, grid, stream);
-            break;
-        case 8: launch_variant<8, 4>(k, grid, stream); break;
-        case 4: launch_variant<4, 4>(k, grid, stream); break;
-        case 2: launch_variant<2, 4>(k, grid, stream); break;
-        default: launch_variant<1, 4>(k, grid, stream); break;
-        }
+        if (lut.m > 7) launch_tn<true>(pl.TN, pl.WR, k, grid, stream);
+        else launch_tn<false>(pl.TN, pl.WR, k, grid, stream);
         AMSIM_HIP_CHECK(hipGetLastError());
         if (nsplit > 1) {
             const int64_t nrows = std::min(row_end, d.R) - row_base;

@@ -25,7 +25,9 @@ int fail(int status, const std::string &msg);
 // Device images of one mantissa-product table.
 //   img_ab[(ma << m) | mb]  one byte per entry: carry << 7 | mantissa << (7 - m)
 //   img_ba[(mb << m) | ma]  the same table transposed
-// (m <= 7 only; both are padded to a multiple of 16 bytes), and
+// (m <= 7 only; both are padded to a multiple of 16 bytes; staged into LDS),
+//   img16_ab / img16_ba     the same with 16-bit entries for 8 <= m <= 11
+// (gathered from global memory), and
 //   lut32[(ma << m) | mb]   carry << 23 | mantissa << (23 - m)   (every m)
 struct Lut {
     int m = 0;
@@ -34,7 +36,10 @@ struct Lut {
     uint8_t *img_ab = nullptr;
     uint8_t *img_ba = nullptr;
     uint32_t *lut32 = nullptr;
-    uint32_t *lut32_t = nullptr;  // transposed 32-bit table (m > 7 path)
+    uint32_t *lut32_t = nullptr;  // transposed 32-bit table
+    // m > 7 only: carry << 15 | mantissa << (15 - m), and its transpose
+    uint16_t *img16_ab = nullptr;
+    uint16_t *img16_ba = nullptr;
 };
 
 }  // namespace amsim

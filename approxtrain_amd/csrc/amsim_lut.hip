@@ -55,6 +55,19 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
         AMSIM_HIP_CHECK(hipMalloc(&l.img_ba, padded));
         AMSIM_HIP_CHECK(hipMemcpy(l.img_ba, ba.data(), padded, hipMemcpyHostToDevice));
     }
+    if (m > 7) {
+        std::vector<uint16_t> ab(total), ba(total);
+        for (size_t i = 0; i < n; ++i)
+            for (size_t j = 0; j < n; ++j) {
+                const uint16_t b = (uint16_t)((carry[i * n + j] << 15) | (mant[i * n + j] << (15 - m)));
+                ab[i * n + j] = b;
+                ba[j * n + i] = b;
+            }
+        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ab, total * 2));
+        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ab, ab.data(), total * 2, hipMemcpyHostToDevice));
+        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ba, total * 2));
+        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ba, ba.data(), total * 2, hipMemcpyHostToDevice));
+    }
     *out = l;
     return AMSIM_OK;
 }
@@ -96,6 +109,8 @@ void lut_free(Lut &l)
     if (l.img_ba) (void)hipFree(l.img_ba);
     if (l.lut32) (void)hipFree(l.lut32);
     if (l.lut32_t) (void)hipFree(l.lut32_t);
+    if (l.img16_ab) (void)hipFree(l.img16_ab);
+    if (l.img16_ba) (void)hipFree(l.img16_ba);
     l = Lut{};
 }
 

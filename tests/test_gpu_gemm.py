@@ -198,3 +198,24 @@ def test_dense_grad_operand_order(amd):
     dx_ref, dw_ref = cpu.dense_grad(cpu.expand_u8(tab, 3), 3, dy, x, w)
     assert np.array_equal(host(dx).view(np.uint32), dx_ref.view(np.uint32))
     assert np.array_equal(host(dw).view(np.uint32), dw_ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("kind", ["MBM", "MIT"])
+@pytest.mark.parametrize("m", [9, 11])
+def test_gemm_wide_mantissa_lut_gathered_from_global_memory(amd, kind, m):
+    """Mantissa widths above 7 (the 2^22-entry m = 11 table does not fit the
+    LDS): 32-bit legacy entries in, LUT gathered through L2.  No reference
+    file or model exists for these widths; the table comes from the oracle's
+    generator (closed-form rules that reproduce every m <= 7 file)."""
+    from approxtrain_amd import ApproxMulLut
+    _set_split(0)
+    img = cpu.lutgen32(kind, m)
+    legacy = (((img >> 23) << 31) | (img & 0x7fffff)).astype(np.uint32)
+    lut = ApproxMulLut.from_entries(legacy, m)
+    rng = np.random.default_rng(80 + m)
+    for (M, N, K, ta, tb) in [(130, 70, 96, 0, 0), (64, 16, 40, 1, 0), (20, 200, 64, 0, 1)]:
+        A, B = _ops(rng, M, N, K, ta, tb)
+        A[0, 0] = np.float32(1e-40)  # one flagged chunk takes the exact path
+        got = host(amd.gemm(lut, dev(A), dev(B), trans_a=bool(ta), trans_b=bool(tb)))
+        want = cpu.gemm(img, m, A, B, transA=ta, transB=tb)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
