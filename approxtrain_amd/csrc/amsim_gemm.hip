@@ -18,10 +18,14 @@
 //     source allows) loads -- dense, im2col-style patches, or filter-gradient
 //     gathers computed on the fly: no im2col / flipped-filter temporaries in
 //     HBM -- in a [k/4][r][4] layout that a lane reads back 16 bytes at a time.
-//   * per MAC: v_or (LUT address), ds_read_u8, v_mul (2^ea * 2^eb),
-//     v_lshl_add (byte -> 1.mant * 2^carry as a float), v_fma (accumulate).
-//     t * f is exact (power of two times an 8-bit significand), so the fused
+//   * per MAC: v_or (LUT address), ds_read_u8, v_lshl_add (LUT byte shifted
+//     into the mantissa/carry position PLUS the uniform operand's sign|exponent
+//     bits = q_pow2 * 1.mant * 2^carry as a float), v_fma with the lane
+//     operand's power of two (accumulate).  The product inside the fma is
+//     exact (power of two times an 8-bit significand), so the fused
 //     multiply-add rounds exactly like the reference's product-then-add.
+//     Zero uniform operands select an all-zero LUT row, zero lane operands a
+//     zero multiplier: no zero test in the loop.
 //   * operands outside the "safe" range (subnormal, inf, NaN, |x| < 2^-63 or
 //     >= 2^64) flag their 32-deep k chunk; flagged chunks take the exact
 //     full-domain product instead (wave-uniform branch), so results are
@@ -39,7 +43,7 @@ constexpr int KG = 4;         // reduction rows handled per scalar-load batch
 constexpr int NG = KC / KG;
 constexpr int QT = 16;        // columns per tile of the pre-decoded uniform operand
 constexpr int WG_THREADS = 256;
-constexpr int LUT_LDS_BYTES = 16384;
+constexpr int LUT_LDS_BYTES = 16384 + 128;   // 2^(2m) entries + one all-zero row of 2^m entries (m <= 7)
 constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels are compiled for
 constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
 constexpr int DEVICE_CUS = 256;               // MI355X; only steers work splitting, never correctness
@@ -125,7 +129,9 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
             }
         }
         unsafe |= operand_unsafe(raw) ? 1 : 0;
-        const uint32_t mant = (raw & 0x7fffffu) >> (23 - a.m);
+        // zero (and padding) elements select the all-zero LUT row that follows the table:
+        // their product term is then exactly +-0 without a test in the inner loop
+        const uint32_t mant = (raw & 0x7fffffffu) ? ((raw & 0x7fffffu) >> (23 - a.m)) : (1u << a.m);
         qw[kk * QT + jj] = (raw & 0xff800000u) | (mant << a.m);
         qraw[kk * QT + jj] = raw;
     }
@@ -453,7 +459,7 @@ void lutgemm_kernel(KArgs a)
 #pragma unroll
                 for (int r = 0; r < KG; ++r) {
                     // keep each row's scalar unpacking next to its use: without the fence the
-                    // scheduler hoists all 128 s_and results to the loop top and spills them
+                    // scheduler hoists every s_and result to the loop top and spills them
                     __builtin_amdgcn_sched_barrier(0);
                     const float ta = u2f(praw[r] & 0xff800000u);
                     const uint32_t ia = __builtin_amdgcn_ubfe(praw[r], (uint32_t)mshift, (uint32_t)m);
@@ -465,9 +471,9 @@ void lutgemm_kernel(KArgs a)
                     }
 #pragma unroll
                     for (int j = 0; j < TN; ++j) {
-                        const float t = u2f(qv[r][j] & 0xff800000u) * ta;
-                        const float f = u2f((L[j] << ESHIFT) + 0x3f800000u);
-                        acc[j] = __builtin_fmaf(t, f, acc[j]);
+                        // (entry << shift) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly
+                        const float g = u2f((L[j] << ESHIFT) + (qv[r][j] & 0xff800000u));
+                        acc[j] = __builtin_fmaf(ta, g, acc[j]);
                     }
                 }
                 qrow += KG * QT;
@@ -583,7 +589,7 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
         const int64_t main_tiles = full_rounds * WG_SLOTS / wgs_per_rowtile;
         const int64_t tail_wgs = (rowtiles - main_tiles) * wgs_per_rowtile;
         if (full_rounds >= 1 && tail_wgs > 0 && tail_wgs * 2 <= WG_SLOTS) {
-            int ts = (int)std::min<int64_t>(WG_SLOTS / tail_wgs, pl.nchunks / 2);
+            int ts = (int)std::min<int64_t>(WG_SLOTS / tail_wgs, pl.nchunks);
             if (ts >= 2) {
                 pl.rows_main = main_tiles * rows;
                 pl.tail_chunks_per_split = (pl.nchunks + ts - 1) / ts;
@@ -682,7 +688,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.p = d.p;
     if (lut.m <= 7) ka.lut_img = d.lane_first ? lut.img_ba : lut.img_ab;
     else ka.lut_img = reinterpret_cast<const uint8_t *>(d.lane_first ? lut.img16_ba : lut.img16_ab);
-    ka.lut_bytes = (int)(((size_t)1 << (2 * lut.m)) + 15) / 16 * 16;
+    ka.lut_bytes = (int)(((size_t)1 << (2 * lut.m)) + ((size_t)1 << lut.m) + 15) / 16 * 16;
     ka.m = lut.m;
     ka.lane_first = d.lane_first ? 1 : 0;
     ka.qw = qa.qw; ka.qraw = qa.qraw; ka.qflags = qa.qflags;

@@ -42,7 +42,8 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
     AMSIM_HIP_CHECK(hipMalloc(&l.lut32_t, total * 4));
     AMSIM_HIP_CHECK(hipMemcpy(l.lut32_t, l32t.data(), total * 4, hipMemcpyHostToDevice));
     if (m <= 7) {
-        const size_t padded = (total + 15) / 16 * 16;
+        // + one all-zero row of n entries after the table (selected by zero operands)
+        const size_t padded = (total + n + 15) / 16 * 16;
         std::vector<uint8_t> ab(padded, 0), ba(padded, 0);
         for (size_t i = 0; i < n; ++i)
             for (size_t j = 0; j < n; ++j) {
@@ -56,17 +57,17 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
         AMSIM_HIP_CHECK(hipMemcpy(l.img_ba, ba.data(), padded, hipMemcpyHostToDevice));
     }
     if (m > 7) {
-        std::vector<uint16_t> ab(total), ba(total);
+        std::vector<uint16_t> ab(total + n, 0), ba(total + n, 0);  // + the all-zero row
         for (size_t i = 0; i < n; ++i)
             for (size_t j = 0; j < n; ++j) {
                 const uint16_t b = (uint16_t)((carry[i * n + j] << 15) | (mant[i * n + j] << (15 - m)));
                 ab[i * n + j] = b;
                 ba[j * n + i] = b;
             }
-        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ab, total * 2));
-        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ab, ab.data(), total * 2, hipMemcpyHostToDevice));
-        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ba, total * 2));
-        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ba, ba.data(), total * 2, hipMemcpyHostToDevice));
+        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ab, (total + n) * 2));
+        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ab, ab.data(), (total + n) * 2, hipMemcpyHostToDevice));
+        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ba, (total + n) * 2));
+        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ba, ba.data(), (total + n) * 2, hipMemcpyHostToDevice));
     }
     *out = l;
     return AMSIM_OK;

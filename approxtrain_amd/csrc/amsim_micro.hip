@@ -12,7 +12,9 @@ constexpr int MICRO_THREADS = 256;
 constexpr int MICRO_UNROLL = 16;
 
 // VMODE 0: v_fma_f32   1: v_add_u32   2: v_lshl_add_u32   3: v_mul_f32
-//       4: the GEMM's per-MAC mix (add, mul, lshl_add, fma) -- 4 ops per slot
+//       4: a 4-op mix (add, mul, lshl_add, fma)
+//       5: the GEMM's per-MAC mix: v_or_b32 (SGPR | VGPR), v_lshl_add_u32 (VGPR << 16 + SGPR),
+//          v_fma_f32 -- 3 ops per slot
 template <int VMODE>
 __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, float *sink, long long *clk)
 {
@@ -28,7 +30,12 @@ __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, fl
             else if (VMODE == 1) asm volatile("v_add_u32 %0, %0, %1" : "+v"(a[j]) : "v"(c1));
             else if (VMODE == 2) asm volatile("v_lshl_add_u32 %0, %0, 16, %1" : "+v"(a[j]) : "v"(c1));
             else if (VMODE == 3) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(a[j]) : "v"(c1));
-            else {
+            else if (VMODE == 5) {
+                float t;
+                asm volatile("v_or_b32 %0, %1, %2" : "=v"(t) : "s"(iters), "v"(c1));
+                asm volatile("v_lshl_add_u32 %0, %1, 16, %2" : "=v"(t) : "v"(t), "s"(iters));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j]) : "v"(c2), "v"(t));
+            } else {
                 float t, f;
                 asm volatile("v_add_u32 %0, %1, %2" : "=v"(t) : "v"(a[j]), "v"(c1));
                 asm volatile("v_mul_f32 %0, %1, %2" : "=v"(f) : "v"(c2), "v"(c1));
@@ -113,7 +120,7 @@ int amsim_calibration_copy(const float *src, float *dst, size_t n, void *stream)
 }
 
 // Runs micro-kernel `kind` (0 = VALU FMA, 1..6 = LDS gather modes 0..5,
-// 10..14 = VALU modes 0..4 with `sink[512..]` receiving the shader-clock ticks
+// 10..15 = VALU modes 0..5 with `sink[512..]` receiving the shader-clock ticks
 // of one workgroup's loop) with
 // `blocks` workgroups of 256 threads, `iters` loop trips of 16 operations per
 // lane, `reps` launches; returns the mean milliseconds per launch measured
@@ -122,7 +129,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
                      double *ops_per_launch)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (kind < 0 || (kind > 6 && kind < 10) || kind > 14 || blocks < 1 || iters < 1 || reps < 1 || !sink || !ms_per_launch || !ops_per_launch)
+    if (kind < 0 || (kind > 6 && kind < 10) || kind > 15 || blocks < 1 || iters < 1 || reps < 1 || !sink || !ms_per_launch || !ops_per_launch)
         return fail(AMSIM_ERR_INVALID, "bad microbench arguments");
     hipEvent_t e0, e1;
     AMSIM_HIP_CHECK(hipEventCreate(&e0));
@@ -135,6 +142,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
         case 12: micro_valu_kernel<2><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 13: micro_valu_kernel<3><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 14: micro_valu_kernel<4><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
+        case 15: micro_valu_kernel<5><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 1: micro_lds_kernel<0><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
         case 2: micro_lds_kernel<1><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
         case 3: micro_lds_kernel<2><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
@@ -154,7 +162,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
     AMSIM_HIP_CHECK(hipEventDestroy(e1));
     AMSIM_HIP_CHECK(hipGetLastError());
     *ms_per_launch = (double)ms / reps;
-    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4 : 1);
+    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4 : kind == 15 ? 3 : 1);
     return AMSIM_OK;
 }
 

@@ -26,7 +26,7 @@ METRIC = "approx GMAC/s + % VALU/LDS roofline, AMConv2D fwd+bwd ResNet-50 3x3, M
 LUT_FILE = os.path.join(ROOT, "tests", "golden", "lut", "MBM_7.bin")
 XS, WS = (32, 56, 56, 64), (3, 3, 64, 64)
 MACS_PER_PASS = 32 * 56 * 56 * 64 * 3 * 3 * 64  # 3 699 376 128
-VALU_OPS_PER_MAC = 4      # v_add (LUT address), v_mul, v_lshl_add, v_fma in the kernel's inner loop
+VALU_OPS_PER_MAC = 3      # v_or (LUT address), v_lshl_add (byte -> product factor), v_fma in the kernel's inner loop
 NOMINAL_OPS_PER_MAC = 5   # the figure the roofline definition quotes as nominal
 
 
@@ -46,7 +46,7 @@ def measure_peaks(lib, cus):
     import torch
     sink = torch.zeros(1024, device="cuda")
     out = {}
-    for name, kind in (("valu_mix_lane_ops_per_s", 14), ("valu_fma_lane_ops_per_s", 10),
+    for name, kind in (("valu_mix_lane_ops_per_s", 15), ("valu_fma_lane_ops_per_s", 10),
                        ("lds_u8_row_gathers_per_s", 1), ("lds_u8_scattered_gathers_per_s", 2)):
         best = 0.0
         for _ in range(3):

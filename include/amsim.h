@@ -154,8 +154,10 @@ int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, i
  * with few outputs split the reduction across workgroups. */
 int amsim_set_split_k(int mode);
 /* Micro-kernels that measure, on the current device, the VALU issue rate
- * (kind 0: independent FP32 FMAs) and the LDS gather rate (kinds 1..6: u8 /
- * u16 / b32 reads, lanes inside one 128-element row or scattered).  Launches
+ * (kind 0 / 10: independent FP32 FMAs; 11..13: v_add_u32, v_lshl_add_u32,
+ * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's 3-op per-MAC mix) and
+ * the LDS gather rate (kinds 1..6: u8 / u16 / b32 reads, lanes inside one
+ * 128-element row or scattered).  Launches
  * `reps` times on `stream`, timed with HIP events; `sink` is any device buffer
  * of >= 256 floats. */
 int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream, float *sink,
