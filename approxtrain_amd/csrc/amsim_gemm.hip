@@ -133,7 +133,7 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
         // their product term is then exactly +-0 without a test in the inner loop
         const uint32_t mant = (raw & 0x7fffffffu) ? ((raw & 0x7fffffu) >> (23 - a.m)) : (1u << a.m);
         qw[kk * QT + jj] = (raw & 0xff800000u) | (mant << a.m);
-        qraw[kk * QT + jj] = raw;
+        qraw[kk * QT + jj] = raw;  // the exact path of a chunk flagged by EITHER operand reads these
     }
     const int any = __any(unsafe);
     if (lane == 0) a.qflags[((size_t)qb * ntiles + jt) * a.nchunks + ch] = (uint32_t)any;
@@ -458,9 +458,9 @@ void lutgemm_kernel(KArgs a)
                 const uint32_t praw[KG] = {p4.x, p4.y, p4.z, p4.w};
 #pragma unroll
                 for (int r = 0; r < KG; ++r) {
-                    // keep each row's scalar unpacking next to its use: without the fence the
-                    // scheduler hoists every s_and result to the loop top and spills them
-                    __builtin_amdgcn_sched_barrier(0);
+                    // 256-row workgroups carry more live scalars: fence each row so the scheduler does
+                    // not hoist every s_and result to the loop top and spill them
+                    if (WR != 1) __builtin_amdgcn_sched_barrier(0);
                     const float ta = u2f(praw[r] & 0xff800000u);
                     const uint32_t ia = __builtin_amdgcn_ubfe(praw[r], (uint32_t)mshift, (uint32_t)m);
                     uint32_t L[TN];
