@@ -1,0 +1,134 @@
+"""Edge cases of the C-ABI entry points on the GPU: empty and ragged
+extents, unaligned operands (scalar staging fallback), workspace errors,
+large strides, reductions that are not multiples of the staging depth."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu
+from tests.gpu_util import dev, host, lut32
+from tests.util import lut_path
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _unsplit():
+    import approxtrain_amd
+    lib = approxtrain_amd.load_library()
+    lib.amsim_set_split_k(0)
+    yield
+    lib.amsim_set_split_k(1)
+
+
+def test_empty_extents_return_empty_outputs():
+    from approxtrain_amd import ApproxMulLut, functors
+    lut = ApproxMulLut.cached(lut_path("MBM", 7))
+    z = lambda *s: torch.zeros(*s, device="cuda")
+    assert functors.gemm(lut, z(0, 5), z(5, 3)).shape == (0, 3)
+    assert functors.gemm(lut, z(4, 5), z(5, 0)).shape == (4, 0)
+    out = functors.gemm(lut, z(4, 0), z(0, 3))
+    assert out.shape == (4, 3) and float(out.abs().sum()) == 0.0
+    assert functors.convam(lut, z(0, 8, 8, 4), z(3, 3, 4, 5), (1, 1), "SAME").shape == (0, 8, 8, 5)
+    assert functors.convam(lut, z(2, 2, 2, 4), z(3, 3, 4, 5), (1, 1), "VALID").shape == (2, 0, 0, 5)  # filter larger than input
+    assert functors.convam_input_grad(lut, (0, 8, 8, 4), z(3, 3, 4, 5), z(0, 8, 8, 5), (1, 1), "SAME").shape == (0, 8, 8, 4)
+    dw = functors.convam_filter_grad(lut, z(0, 8, 8, 4), (3, 3, 4, 5), z(0, 8, 8, 5), (1, 1), "SAME")
+    assert dw.shape == (3, 3, 4, 5) and float(dw.abs().sum()) == 0.0  # empty reduction -> zeros
+    assert functors.denseam(lut, z(0, 7), z(7, 3)).shape == (0, 3)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (63, 15, 31), (65, 17, 33), (64, 16, 32), (129, 1, 95), (2, 300, 3)])
+def test_ragged_extents(M, N, K):
+    from approxtrain_amd import ApproxMulLut, functors
+    rng = np.random.default_rng(M + N + K)
+    A, B = rng.standard_normal((M, K)).astype(np.float32), rng.standard_normal((K, N)).astype(np.float32)
+    got = host(functors.gemm(ApproxMulLut.cached(lut_path("MBM", 7)), dev(A), dev(B)))
+    assert np.array_equal(got.view(np.uint32), cpu.gemm(lut32("MBM", 7), 7, A, B).view(np.uint32))
+
+
+def test_unaligned_operands_use_scalar_staging():
+    """Operands that start 4 bytes into an allocation are not 16-byte aligned:
+    the float4 staging path must not be taken (and results stay bit-equal)."""
+    from approxtrain_amd import ApproxMulLut, functors
+    lut = ApproxMulLut.cached(lut_path("MBM", 7))
+    L = lut32("MBM", 7)
+    rng = np.random.default_rng(5)
+    M, N, K = 96, 48, 64
+    A, B = rng.standard_normal((M, K)).astype(np.float32), rng.standard_normal((K, N)).astype(np.float32)
+    buf = torch.zeros(M * K + 1, device="cuda")
+    buf[1:] = dev(A).flatten()
+    Au = buf[1:].view(M, K)
+    assert Au.data_ptr() % 16 != 0 and Au.is_contiguous()
+    got = host(functors.gemm(lut, Au, dev(B)))
+    assert np.array_equal(got.view(np.uint32), cpu.gemm(L, 7, A, B).view(np.uint32))
+    xs, ws = (2, 6, 6, 8), (3, 3, 8, 12)
+    x, w = rng.standard_normal(xs).astype(np.float32), rng.standard_normal(ws).astype(np.float32)
+    xb = torch.zeros(int(np.prod(xs)) + 1, device="cuda")
+    xb[1:] = dev(x).flatten()
+    xu = xb[1:].view(*xs)
+    got = host(functors.convam(lut, xu, dev(w), (1, 1), "SAME"))
+    assert np.array_equal(got.view(np.uint32), cpu.conv2d_fwd(L, 7, x, w, (1, 1), "SAME").view(np.uint32))
+
+
+def test_leading_dimension_larger_than_row_and_workspace_errors():
+    import approxtrain_amd
+    from approxtrain_amd import ApproxMulLut
+    lib = approxtrain_amd.load_library()
+    lut = ApproxMulLut.cached(lut_path("MBM", 7))
+    rng = np.random.default_rng(6)
+    M, N, K, lda, ldb, ldc = 70, 20, 40, 48, 28, 24
+    A = rng.standard_normal((M, lda)).astype(np.float32)
+    B = rng.standard_normal((K, ldb)).astype(np.float32)
+    Ad, Bd = dev(A), dev(B)
+    Cd = torch.full((M, ldc), 7.0, device="cuda")
+    nbytes = lib.amsim_gemm_workspace_bytes(0, 0, M, N, K, 1)
+    ws = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda")
+    base = ws.data_ptr() + (-ws.data_ptr()) % 256
+    args = lambda wsp, wsb: (lut.handle, 0, 0, 0, M, N, K, C.c_void_p(Ad.data_ptr()), lda, C.c_void_p(Bd.data_ptr()),
+                             ldb, C.c_void_p(Cd.data_ptr()), ldc, 1, 0, 0, 0, C.c_void_p(wsp), wsb, None)
+    assert lib.amsim_gemm_f32(*args(base, nbytes)) == 0
+    got = host(Cd)
+    want = cpu.gemm(lut32("MBM", 7), 7, A[:, :K].copy(), B[:, :N].copy())
+    assert np.array_equal(got[:, :N].view(np.uint32), want.view(np.uint32))
+    assert (got[:, N:] == 7.0).all()  # padding columns of C untouched
+    assert lib.amsim_gemm_f32(*args(base, nbytes - 1)) == 5        # too small
+    assert lib.amsim_gemm_f32(*args(base + 4, nbytes)) == 5        # misaligned
+    assert lib.amsim_gemm_f32(*args(0, 0)) == 5                    # missing
+    assert b"workspace" in lib.amsim_last_error()
+    bad = list(args(base, nbytes)); bad[8] = K - 1                 # lda < K
+    assert lib.amsim_gemm_f32(*bad) == 1
+
+
+@pytest.mark.parametrize("stride", [3, 4])
+def test_conv_large_strides_and_asymmetric_shapes(stride):
+    from approxtrain_amd import ApproxMulLut, functors
+    lut = ApproxMulLut.cached(lut_path("MIT", 7))
+    L = lut32("MIT", 7)
+    rng = np.random.default_rng(stride)
+    xs, ws = (2, 17, 13, 4), (5, 2, 4, 9)
+    x, w = rng.standard_normal(xs).astype(np.float32), rng.standard_normal(ws).astype(np.float32)
+    for padding in ("SAME", "VALID"):
+        st = (stride, stride)
+        want = cpu.conv2d_fwd(L, 7, x, w, st, padding)
+        dy = rng.standard_normal(want.shape).astype(np.float32)
+        assert np.array_equal(host(functors.convam(lut, dev(x), dev(w), st, padding)).view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(host(functors.convam_input_grad(lut, xs, dev(w), dev(dy), st, padding)).view(np.uint32),
+                              cpu.conv2d_grad_input(L, 7, xs, w, dy, st, padding).view(np.uint32))
+        assert np.array_equal(host(functors.convam_filter_grad(lut, dev(x), ws, dev(dy), st, padding)).view(np.uint32),
+                              cpu.conv2d_grad_filter(L, 7, x, ws, dy, st, padding).view(np.uint32))
+
+
+def test_runs_on_a_non_default_stream():
+    from approxtrain_amd import ApproxMulLut, functors
+    lut = ApproxMulLut.cached(lut_path("MBM", 7))
+    rng = np.random.default_rng(9)
+    A, B = rng.standard_normal((200, 96)).astype(np.float32), rng.standard_normal((96, 80)).astype(np.float32)
+    s = torch.cuda.Stream()
+    Ad, Bd = dev(A), dev(B)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        out = functors.gemm(lut, Ad, Bd)
+    s.synchronize()
+    assert np.array_equal(host(out).view(np.uint32), cpu.gemm(lut32("MBM", 7), 7, A, B).view(np.uint32))
