@@ -23,6 +23,21 @@ __device__ __forceinline__ bool operand_unsafe(uint32_t bits)
     return mag != 0u && (e - 64u) > 126u;
 }
 
+// Range bookkeeping for many operands at once (two min/max updates per operand
+// instead of a compare chain): t = bits << 1 drops the sign; zeros wrap to the
+// top of the range in (t - 1) and so never lower the minimum.
+struct SafeRange {
+    uint32_t tmax = 0u, tmin = 0xffffffffu;
+    __device__ __forceinline__ void add(uint32_t bits)
+    {
+        const uint32_t t = bits << 1;
+        tmax = max(tmax, t);
+        tmin = min(tmin, t - 1u);
+    }
+    // same predicate as operand_unsafe() over everything added
+    __device__ __forceinline__ bool unsafe() const { return tmax >= (191u << 24) || tmin < (64u << 24) - 1u; }
+};
+
 // Full-domain product.  `entry16` is the LUT byte (carry << 7 | mantissa
 // left-aligned in 7 bits) shifted left by 16, i.e. carry << 23 | mantissa.
 // Restates the exponent / special-case logic of the C functional models:

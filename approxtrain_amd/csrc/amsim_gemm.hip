@@ -300,10 +300,21 @@ void lutgemm_kernel(KArgs a)
         }
     };
 
+    // Filter-gradient tiles that lie inside one (fy, fx) (channel count a multiple of the tile
+    // height, tile fully inside R): wave-uniform window offset
+    const bool gf_uniform = PK == P_GF && (a.p.C % ROWS == 0) && row0 + ROWS <= a.R;
+    int gf_fy = 0, gf_fx = 0, gf_c0 = 0;
+    if (gf_uniform) {
+        gf_c0 = (int)(row0 % a.p.C);
+        const int t = (int)(row0 / a.p.C);
+        gf_fx = t % a.p.KW;
+        gf_fy = t / a.p.KW;
+    }
+
     uint32_t pv[ELEMS];
     auto load_chunk = [&](int ch) -> int {
         const int64_t k0 = (int64_t)ch * KC;
-        int unsafe = 0;
+        SafeRange sr;
         if (STAGE == STAGE_K4) {
             // thread -> (row, quad of 4 consecutive k); all four share (fy, fx) because C % 4 == 0
             const int kq = (tid & (KC / 4 - 1)) * 4;
@@ -334,7 +345,7 @@ void lutgemm_kernel(KArgs a)
                     }
                 }
                 pv[4 * i + 0] = v.x; pv[4 * i + 1] = v.y; pv[4 * i + 2] = v.z; pv[4 * i + 3] = v.w;
-                unsafe |= (operand_unsafe(v.x) | operand_unsafe(v.y) | operand_unsafe(v.z) | operand_unsafe(v.w)) ? 1 : 0;
+                sr.add(v.x); sr.add(v.y); sr.add(v.z); sr.add(v.w);
             }
             if (PK == P_DENSE) dptr += dchunk;
         } else if (PK == P_DENSE) {
@@ -349,7 +360,7 @@ void lutgemm_kernel(KArgs a)
                     if (k0 + kk < a.K && drow < dvalid_rows) v = f2u(dptr[(int64_t)i * dstep]);
                 }
                 pv[i] = v;
-                unsafe |= operand_unsafe(v) ? 1 : 0;
+                sr.add(v);
             }
             dptr += dchunk;
         } else if (PK == P_PATCH) {  // STAGE_K: this thread's k is fixed for the chunk
@@ -374,7 +385,7 @@ void lutgemm_kernel(KArgs a)
                     if (on_grid) v = f2u(pbase[ri.x + (sy_ * a.p.SW + sx_) * a.p.C + c]);
                 }
                 pv[i] = v;
-                unsafe |= operand_unsafe(v) ? 1 : 0;
+                sr.add(v);
             }
         } else {  // P_GF, staged along r: this thread stages ELEMS consecutive k (pixels) of its row
             const int rl = tid & (ROWS - 1);
@@ -385,22 +396,37 @@ void lutgemm_kernel(KArgs a)
             const int64_t t = kfirst / a.p.GW;
             int y = (int)(t % a.p.GH);
             int b = (int)(t / a.p.GH);
+            if (gf_uniform) {
+                // all rows of the tile share (fy, fx): the bounds test is wave-uniform and the
+                // address is a scalar pixel offset plus this lane's channel
 #pragma unroll
-            for (int i = 0; i < ELEMS; ++i) {
-                uint32_t v = 0;
-                if (kfirst + i < a.K) {
-                    const int iy0 = y * a.p.sy - a.p.pt, ix0 = x * a.p.sx - a.p.pl;
-                    const int iy = iy0 + ri.y, ix = ix0 + ri.z;
-                    if ((unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
-                        v = f2u(pbase[((b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + ri.x]);
+                for (int i = 0; i < ELEMS; ++i) {
+                    uint32_t v = 0;
+                    const int iy = y * a.p.sy - a.p.pt + gf_fy, ix = x * a.p.sx - a.p.pl + gf_fx;
+                    if (kfirst + i < a.K && (unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
+                        v = f2u(pbase[((b * a.p.SH + iy) * a.p.SW + ix) * a.p.C + gf_c0 + rl]);
+                    pv[i] = v;
+                    sr.add(v);
+                    if (++x == a.p.GW) { x = 0; if (++y == a.p.GH) { y = 0; ++b; } }
                 }
-                pv[i] = v;
-                unsafe |= operand_unsafe(v) ? 1 : 0;
-                if (++x == a.p.GW) { x = 0; if (++y == a.p.GH) { y = 0; ++b; } }
+            } else {
+#pragma unroll
+                for (int i = 0; i < ELEMS; ++i) {
+                    uint32_t v = 0;
+                    if (kfirst + i < a.K) {
+                        const int iy0 = y * a.p.sy - a.p.pt, ix0 = x * a.p.sx - a.p.pl;
+                        const int iy = iy0 + ri.y, ix = ix0 + ri.z;
+                        if ((unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
+                            v = f2u(pbase[((b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + ri.x]);
+                    }
+                    pv[i] = v;
+                    sr.add(v);
+                    if (++x == a.p.GW) { x = 0; if (++y == a.p.GH) { y = 0; ++b; } }
+                }
             }
         }
         if (PK == P_PATCH) advance_chunk_base();
-        return unsafe;
+        return sr.unsafe() ? 1 : 0;
     };
     auto store_chunk = [&]() {
         if (STAGE == STAGE_K4) {
