@@ -53,6 +53,7 @@ constexpr int TARGET_WAVES = WG_SLOTS * 4;
 static std::atomic<int> g_split_k{1};
 
 typedef const __attribute__((address_space(4))) uint32_t *cq1_t;
+typedef const __attribute__((address_space(4))) uint64_t *cq2_t;
 
 // staging modes of the lane operand
 enum { STAGE_R = 0,   // threads run along r, one element each (source contiguous in r)
@@ -475,30 +476,37 @@ void lutgemm_kernel(KArgs a)
             cq1_t qrow = qw + qoff;
 #pragma unroll 1
             for (int g = 0; g < NG; ++g) {
-                uint32_t qv[KG][TN];
+                // column pairs are unpacked with 64-bit scalar ops: half the SALU instructions
+                constexpr int TN2 = (TN + 1) / 2;
+                uint64_t qw2[KG][TN2];
 #pragma unroll
                 for (int r = 0; r < KG; ++r)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) qv[r][j] = qrow[r * QT + j];
+                    for (int j = 0; j < TN2; ++j) {
+                        if (TN >= 2) qw2[r][j] = reinterpret_cast<cq2_t>(qrow + r * QT)[j];
+                        else qw2[r][j] = qrow[r * QT];
+                    }
                 const uint4 p4 = Pt4[g * GS + lrow];
                 const uint32_t praw[KG] = {p4.x, p4.y, p4.z, p4.w};
 #pragma unroll
                 for (int r = 0; r < KG; ++r) {
                     // 256-row workgroups carry more live scalars: fence each row so the scheduler does
                     // not hoist every s_and result to the loop top and spill them
-                    if (WR != 1) __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_sched_barrier(0);
                     const float ta = u2f(praw[r] & 0xff800000u);
                     const uint32_t ia = __builtin_amdgcn_ubfe(praw[r], (uint32_t)mshift, (uint32_t)m);
                     uint32_t L[TN];
 #pragma unroll
                     for (int j = 0; j < TN; ++j) {
-                        const uint32_t li = (qv[r][j] & 0x7fffffu) | ia;
+                        const uint64_t qi2 = qw2[r][j >> 1] & 0x007fffff007fffffull;
+                        const uint32_t li = (uint32_t)(qi2 >> (32 * (j & 1))) | ia;
                         L[j] = LUTG ? (uint32_t)lut_g[li] : (uint32_t)lut_s[li];
                     }
 #pragma unroll
                     for (int j = 0; j < TN; ++j) {
                         // (entry << shift) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly
-                        const float g = u2f((L[j] << ESHIFT) + (qv[r][j] & 0xff800000u));
+                        const uint64_t qt2 = qw2[r][j >> 1] & 0xff800000ff800000ull;
+                        const float g = u2f((L[j] << ESHIFT) + (uint32_t)(qt2 >> (32 * (j & 1))));
                         acc[j] = __builtin_fmaf(ta, g, acc[j]);
                     }
                 }
