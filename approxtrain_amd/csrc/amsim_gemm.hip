@@ -142,8 +142,9 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
 
 // ---------------------------------------------------------------------------
 // lane-operand row bookkeeping, kept in LDS: one int4 per local row.
-//   P_PATCH: {source offset of image b, y*sy - pt, x*sx - pl, 0}; rows past the
-//            end get a y origin far outside the source.
+//   P_PATCH: {source offset of image b, y*sy - pt, x*sx - pl, source offset of the
+//            window origin (undilated sources)}; rows past the end get a y origin
+//            far outside the source.
 //   P_GF:    {(fy*SW + fx)*C + c, fy, fx, 0}; rows past the end get fy far outside.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t row0, int rows, int4 *ri)
@@ -157,7 +158,8 @@ __device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t 
                 const int64_t t = r / p.GW;
                 const int y = (int)(t % p.GH);
                 const int b = (int)(t / p.GH);
-                v = make_int4(b * p.SH * p.SW * p.C, y * p.sy - p.pt, x * p.sx - p.pl, 0);
+                const int vy0 = y * p.sy - p.pt, vx0 = x * p.sx - p.pl;
+                v = make_int4(b * p.SH * p.SW * p.C, vy0, vx0, (b * p.SH * p.SW + vy0 * p.SW + vx0) * p.C);
             } else if (p.kind == P_GF) {
                 const int c = (int)(r % p.C);
                 const int t = (int)(r / p.C);
@@ -196,6 +198,7 @@ void lutgemm_kernel(KArgs a)
     constexpr int ESHIFT = LUTG ? 8 : 16;  // LUT entry -> carry << 23 | mantissa
     __shared__ uint4 Pt4[NG * GS];
     __shared__ int4 rowinfo[PK == P_DENSE ? 1 : ROWS];
+    __shared__ uint32_t pflag[2];  // "this chunk's staged tile holds an unsafe operand", by chunk parity
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -226,6 +229,7 @@ void lutgemm_kernel(KArgs a)
         for (int i = tid * 16; i < a.lut_bytes; i += WG_THREADS * 16)
             *reinterpret_cast<uint4 *>(lut_s + i) = *reinterpret_cast<const uint4 *>(a.lut_img + i);
     if (PK != P_DENSE) fill_rowinfo(a.p, a.R, row0, ROWS, rowinfo);
+    if (tid < 2) pflag[tid] = 0u;
     __syncthreads();
 
     const float *pbase = a.p.base + (int64_t)bz * a.p.batch_stride;
@@ -301,6 +305,10 @@ void lutgemm_kernel(KArgs a)
         }
     };
 
+    // Undilated patch sources whose channel count is a multiple of the chunk depth: every
+    // chunk lies inside one filter tap, so the tap offset and the window test are scalar work
+    const bool tap_uniform = PK == P_PATCH && STAGE == STAGE_K4 && a.p.dy == 1 && a.p.dx == 1 && (a.p.C % KC == 0);
+
     // Filter-gradient tiles that lie inside one (fy, fx) (channel count a multiple of the tile
     // height, tile fully inside R): wave-uniform window offset
     const bool gf_uniform = PK == P_GF && (a.p.C % ROWS == 0) && row0 + ROWS <= a.R;
@@ -322,12 +330,17 @@ void lutgemm_kernel(KArgs a)
             const int64_t k = k0 + kq;
             const bool kvalid = k < a.K;  // K % 4 == 0 on this path
             int c = 0, fy = 0, fx = 0;
-            if (PK == P_PATCH) decompose_k(k, kq, c, fx, fy);
+            if (PK == P_PATCH && !tap_uniform) decompose_k(k, kq, c, fx, fy);
+            const int tapoff = (cb_fy * a.p.SW + cb_fx) * a.p.C + cb_c + kq;
 #pragma unroll
             for (int i = 0; i < QUADS; ++i) {
                 const int rl = (tid >> 3) + i * (WG_THREADS / (KC / 4));
                 uint4 v = make_uint4(0, 0, 0, 0);
-                if (PK == P_DENSE) {
+                if (PK == P_PATCH && tap_uniform) {
+                    const int4 ri = rowinfo[rl];
+                    if ((unsigned)(ri.y + cb_fy) < (unsigned)a.p.SH && (unsigned)(ri.z + cb_fx) < (unsigned)a.p.SW)
+                        v = *reinterpret_cast<const uint4 *>(pbase + (ri.w + tapoff));
+                } else if (PK == P_DENSE) {
                     // dptr walks this thread's first row; rows i*32 further down are dstep apart
                     if (kvalid && drow + i * (WG_THREADS / (KC / 4)) < dvalid_rows)
                         v = *reinterpret_cast<const uint4 *>(dptr + (int64_t)i * dstep);
@@ -465,9 +478,26 @@ void lutgemm_kernel(KArgs a)
     const int mshift = 23 - m;
 
     for (int ch = ch_begin; ch < ch_end; ++ch) {
+        // The instruction arbiter favours a SIMD's oldest waves, so left alone the workgroups
+        // that share a CU finish far apart and the last ones run on a mostly empty CU.  Wave
+        // priority falls as a workgroup nears its end (more than 1/2, 1/4, 1/8 of its chunks
+        // left, then the rest): whoever is behind catches up and the CU stays full to the end.
+        {
+            const int n = ch_end - ch_begin, rem = ch_end - ch;
+            if (2 * rem > n) __builtin_amdgcn_s_setprio(3);
+            else if (4 * rem > n) __builtin_amdgcn_s_setprio(2);
+            else if (8 * rem > n) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+        }
         __syncthreads();  // every wave is done with the previous chunk's tile
         store_chunk();
-        const int p_unsafe = __syncthreads_or(unsafe);
+        // Unsafe operands are rare: whoever staged one raises the chunk's flag (slot = chunk
+        // parity); the slot of the previous chunk is cleared for the chunk after this one,
+        // ordered against its writers by the barrier at the top of the next trip.
+        if (unsafe) pflag[ch & 1] = 1u;
+        __syncthreads();
+        const uint32_t p_unsafe = __builtin_amdgcn_readfirstlane(pflag[ch & 1]);
+        if (tid == 0) pflag[(ch & 1) ^ 1] = 0u;
         if (ch + 1 < ch_end) unsafe = load_chunk(ch + 1);  // in flight during the MACs below
         if (!active) continue;
         const uint32_t q_unsafe = qflags[ch];
