@@ -71,13 +71,19 @@ struct KArgs {
     const uint32_t *qflags;  // [qb][Jp/16][nchunks]
     int q_batches;
     int64_t R, J, K;
-    int Jp, nchunks, nsplit, chunks_per_split;
+    int Jp, nchunks;
     float *out;
     int64_t so_r, so_j, out_batch_stride;
-    float *partial;          // [nsplit][batch][Rp][Jp] when nsplit > 1 (rows relative to row_base)
-    int64_t Rp;
-    int64_t row_base;        // first row this launch covers
+    float *partial;          // [nsplit][batch][Rp][Jp] of the segment whose nsplit > 1 (rows relative to its row_base)
     int batch;
+    // A launch covers up to two row segments, workgroups of seg[0] first in dispatch order:
+    // seg[0] the split-reduction tail (if any), seg[1] the main part.
+    struct Seg {
+        int64_t row_base, Rp;        // first row, padded row count
+        int nsplit, chunks_per_split;
+        unsigned X, Y, Z;            // row tiles, column groups, batch x splits
+        unsigned total;              // X * Y * Z
+    } seg[2];
 };
 
 // ---------------------------------------------------------------------------
@@ -171,8 +177,6 @@ __device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t 
     }
 }
 
-__device__ __forceinline__ int ch_begin_of(const KArgs &a, int split) { return split * a.chunks_per_split; }
-
 // ---------------------------------------------------------------------------
 // main kernel
 // ---------------------------------------------------------------------------
@@ -208,10 +212,16 @@ void lutgemm_kernel(KArgs a)
     // XCD has its own L2.  Renumber so that each XCD works on a contiguous run
     // of tiles (row tile fastest, then column group, then split / batch): the
     // workgroups that share uniform-operand tiles and input rows then share an L2.
+    const bool in_first = blockIdx.x < a.seg[0].total;
+    const int64_t seg_row_base = in_first ? a.seg[0].row_base : a.seg[1].row_base;
+    const int64_t seg_Rp = in_first ? a.seg[0].Rp : a.seg[1].Rp;
+    const int seg_nsplit = in_first ? a.seg[0].nsplit : a.seg[1].nsplit;
+    const int seg_cps = in_first ? a.seg[0].chunks_per_split : a.seg[1].chunks_per_split;
     unsigned bx, by, bzz;
     {
-        const unsigned X = gridDim.x, Y = gridDim.y, T = X * Y * gridDim.z;
-        const unsigned L = (blockIdx.z * Y + blockIdx.y) * X + blockIdx.x;
+        const unsigned X = in_first ? a.seg[0].X : a.seg[1].X, Y = in_first ? a.seg[0].Y : a.seg[1].Y;
+        const unsigned T = in_first ? a.seg[0].total : a.seg[1].total;
+        const unsigned L = in_first ? blockIdx.x : blockIdx.x - a.seg[0].total;
         const unsigned xcd = L % NUM_XCD, idx = L / NUM_XCD;
         const unsigned chunk = T / NUM_XCD, rem = T % NUM_XCD;
         const unsigned V = xcd * chunk + (xcd < rem ? xcd : rem) + idx;
@@ -219,8 +229,8 @@ void lutgemm_kernel(KArgs a)
         by = (V / X) % Y;
         bzz = V / (X * Y);
     }
-    const int bz = bzz / a.nsplit, split = bzz % a.nsplit;
-    const int64_t row0 = a.row_base + (int64_t)bx * ROWS;
+    const int bz = bzz / seg_nsplit, split = bzz % seg_nsplit;
+    const int64_t row0 = seg_row_base + (int64_t)bx * ROWS;
     const int j0 = (by * WC + wc) * TN;
     const bool active = j0 < a.J;
     const int m = a.m;
@@ -243,8 +253,8 @@ void lutgemm_kernel(KArgs a)
     const cq1_t qraw = (cq1_t)(uintptr_t)(a.qraw + qtile);
     const cq1_t qflags = (cq1_t)(uintptr_t)(a.qflags + ((size_t)qb * (a.Jp / QT) + (size_t)(j0 / QT)) * a.nchunks);
 
-    const int ch_begin = split * a.chunks_per_split;
-    const int ch_end = min(a.nchunks, ch_begin + a.chunks_per_split);
+    const int ch_begin = split * seg_cps;
+    const int ch_end = min(a.nchunks, ch_begin + seg_cps);
 
     // Dense sources: one per-thread pointer to the first element this thread
     // stages, a uniform step between its successive elements, and a uniform
@@ -274,7 +284,7 @@ void lutgemm_kernel(KArgs a)
         }
         // pin the walking state into vector registers
         asm volatile("" : "+v"(dstep), "+v"(dchunk));
-        dptr += (int64_t)ch_begin_of(a, split) * dchunk;
+        dptr += (int64_t)(split * seg_cps) * dchunk;
     }
 
     // Patch sources: (fy, fx, c) of the first k of the next chunk to stage, walked
@@ -282,7 +292,7 @@ void lutgemm_kernel(KArgs a)
     int cb_c = 0, cb_fx = 0, cb_fy = 0;
     const bool patch_walk = PK == P_PATCH && a.p.C >= KC;
     if (patch_walk) {
-        const int64_t kb = (int64_t)ch_begin_of(a, split) * KC;
+        const int64_t kb = (int64_t)(split * seg_cps) * KC;
         cb_c = (int)(kb % a.p.C);
         const int t = (int)(kb / a.p.C);
         cb_fx = t % a.p.KW;
@@ -562,7 +572,7 @@ void lutgemm_kernel(KArgs a)
 
     const int64_t r = row0 + lrow;
     if (!active) return;
-    if (a.nsplit == 1) {
+    if (seg_nsplit == 1) {
         if (r < a.R) {
             float *o = a.out + (int64_t)bz * a.out_batch_stride + r * a.so_r;
 #pragma unroll
@@ -570,7 +580,7 @@ void lutgemm_kernel(KArgs a)
                 if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = acc[j];
         }
     } else {
-        float *o = a.partial + (((size_t)split * a.batch + bz) * a.Rp + (r - a.row_base)) * a.Jp + j0;
+        float *o = a.partial + (((size_t)split * a.batch + bz) * seg_Rp + (r - seg_row_base)) * a.Jp + j0;
 #pragma unroll
         for (int j = 0; j < TN; ++j) o[j] = acc[j];
     }
@@ -765,34 +775,45 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
 
     const int rows = 64 * pl.WR, wc = 4 / pl.WR;
     const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;
-    const unsigned gy = (unsigned)((jchunks + wc - 1) / wc);
-    if (gy > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "uniform dimension exceeds the grid limit");
+    const int64_t gy = (jchunks + wc - 1) / wc;
 
-    auto launch = [&](int64_t row_base, int64_t row_end, int nsplit, int cps) -> int {
-        KArgs k = ka;
-        k.row_base = row_base;
-        k.nsplit = nsplit;
-        k.chunks_per_split = cps;
-        k.Rp = (row_end - row_base + rows - 1) / rows * rows;
-        const int64_t gz = (int64_t)d.batch * nsplit;
-        if (gz > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch x split-K exceeds the grid limit");
-        dim3 grid((unsigned)(k.Rp / rows), gy, (unsigned)gz);
-        if (lut.m > 7) launch_tn<true>(pl.TN, pl.WR, k, grid, stream);
-        else launch_tn<false>(pl.TN, pl.WR, k, grid, stream);
-        AMSIM_HIP_CHECK(hipGetLastError());
-        if (nsplit > 1) {
-            const int64_t nrows = std::min(row_end, d.R) - row_base;
-            RArgs ra{k.partial, d.out, nrows, d.J, k.Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp, nsplit, d.batch, row_base};
-            dim3 rgrid((unsigned)((nrows * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
-            splitk_reduce_kernel<<<rgrid, WG_THREADS, 0, stream>>>(ra);
-            AMSIM_HIP_CHECK(hipGetLastError());
-        }
-        return AMSIM_OK;
+    // One launch: the split-reduction tail's workgroups (if any) come first in dispatch order
+    // and share the machine with the first main workgroups; the main workgroups that start
+    // after them catch up through wave priority.
+    auto fill_seg = [&](KArgs::Seg &sg, int64_t row_base, int64_t row_end, int nsplit, int cps) -> int64_t {
+        sg.row_base = row_base;
+        sg.Rp = (row_end - row_base + rows - 1) / rows * rows;
+        sg.nsplit = nsplit;
+        sg.chunks_per_split = cps;
+        const int64_t X = sg.Rp / rows, Z = (int64_t)d.batch * nsplit;
+        const int64_t total = X * gy * Z;
+        sg.X = (unsigned)X; sg.Y = (unsigned)gy; sg.Z = (unsigned)Z;
+        sg.total = (unsigned)total;
+        return total;
     };
-    int rc = launch(0, pl.rows_main, pl.nsplit, pl.chunks_per_split);
-    if (rc != AMSIM_OK) return rc;
-    if (pl.rows_main < d.R) rc = launch(pl.rows_main, d.R, pl.tail_nsplit, pl.tail_chunks_per_split);
-    return rc;
+    const bool has_tail = pl.rows_main < d.R;
+    int64_t total = 0;
+    if (has_tail) total += fill_seg(ka.seg[0], pl.rows_main, d.R, pl.tail_nsplit, pl.tail_chunks_per_split);
+    else ka.seg[0] = KArgs::Seg{0, 0, 1, 0, 0, 0, 0, 0};
+    total += fill_seg(ka.seg[1], 0, pl.rows_main, pl.nsplit, pl.chunks_per_split);
+    if (total >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "workgroup count exceeds the grid limit");
+    const dim3 grid((unsigned)total);
+    if (lut.m > 7) launch_tn<true>(pl.TN, pl.WR, ka, grid, stream);
+    else launch_tn<false>(pl.TN, pl.WR, ka, grid, stream);
+    AMSIM_HIP_CHECK(hipGetLastError());
+
+    const KArgs::Seg *split_seg = has_tail && pl.tail_nsplit > 1 ? &ka.seg[0] : pl.nsplit > 1 ? &ka.seg[1] : nullptr;
+    if (split_seg) {
+        if (d.batch > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
+        const int64_t row_end = split_seg == &ka.seg[0] ? d.R : pl.rows_main;
+        const int64_t nrows = row_end - split_seg->row_base;
+        RArgs ra{ka.partial, d.out, nrows, d.J, split_seg->Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp,
+                 split_seg->nsplit, d.batch, split_seg->row_base};
+        dim3 rgrid((unsigned)((nrows * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
+        splitk_reduce_kernel<<<rgrid, WG_THREADS, 0, stream>>>(ra);
+        AMSIM_HIP_CHECK(hipGetLastError());
+    }
+    return AMSIM_OK;
 }
 
 // ---------------------------------------------------------------------------
