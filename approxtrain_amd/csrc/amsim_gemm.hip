@@ -595,24 +595,41 @@ struct RArgs {
     int64_t row_base;
 };
 
+constexpr int RED_OUTS = 64;                      // outputs per workgroup
+constexpr int RED_WAYS = WG_THREADS / RED_OUTS;   // waves that share the splits of one output
+
+// Each wave takes every RED_WAYS-th split of 64 consecutive outputs in eight interleaved
+// chains (eight loads in flight); the chains and then the waves' sums are combined in a
+// fixed order, so the result does not depend on scheduling.
 __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
 {
-    const int64_t idx = (int64_t)blockIdx.x * WG_THREADS + threadIdx.x;
+    __shared__ float part[RED_WAYS][RED_OUTS];
+    const int o = threadIdx.x & (RED_OUTS - 1), way = threadIdx.x / RED_OUTS;
+    const int64_t idx = (int64_t)blockIdx.x * RED_OUTS + o;
     const int bz = blockIdx.y;
-    if (idx >= a.R * a.J) return;
-    const int64_t r = idx / a.J, j = idx - r * a.J;
-    // eight interleaved chains keep eight loads in flight; the combination order is fixed
+    const bool valid = idx < a.R * a.J;
+    int64_t r = 0, j = 0;
     float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const size_t stride = (size_t)a.batch * a.Rp * a.Jp;
-    const float *src = a.partial + ((size_t)bz * a.Rp + r) * a.Jp + j;
-    int sp = 0;
-    for (; sp + 8 <= a.nsplit; sp += 8) {
+    if (valid) {
+        r = idx / a.J;
+        j = idx - r * a.J;
+        const size_t stride = (size_t)a.batch * a.Rp * a.Jp;
+        const float *src = a.partial + ((size_t)bz * a.Rp + r) * a.Jp + j;
+        int sp = way;
+        for (; sp + 7 * RED_WAYS < a.nsplit; sp += 8 * RED_WAYS) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) c[u] += src[(size_t)(sp + u) * stride];
+            for (int u = 0; u < 8; ++u) c[u] += src[(size_t)(sp + u * RED_WAYS) * stride];
+        }
+        for (int u = 0; sp < a.nsplit; sp += RED_WAYS, ++u) c[u] += src[(size_t)sp * stride];
     }
-    for (int u = 0; sp < a.nsplit; ++sp, ++u) c[u] += src[(size_t)sp * stride];
-    const float s = ((c[0] + c[1]) + (c[2] + c[3])) + ((c[4] + c[5]) + (c[6] + c[7]));
-    a.out[(int64_t)bz * a.out_batch_stride + (a.row_base + r) * a.so_r + j * a.so_j] = s;
+    part[way][o] = ((c[0] + c[1]) + (c[2] + c[3])) + ((c[4] + c[5]) + (c[6] + c[7]));
+    __syncthreads();
+    if (way == 0 && valid) {
+        float s = part[0][o];
+#pragma unroll
+        for (int w = 1; w < RED_WAYS; ++w) s += part[w][o];
+        a.out[(int64_t)bz * a.out_batch_stride + (a.row_base + r) * a.so_r + j * a.so_j] = s;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -735,7 +752,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
         RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0};
-        dim3 grid((unsigned)((d.R * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
+        dim3 grid((unsigned)((d.R * d.J + RED_OUTS - 1) / RED_OUTS), (unsigned)d.batch);
         splitk_reduce_kernel<<<grid, WG_THREADS, 0, stream>>>(ra);
         AMSIM_HIP_CHECK(hipGetLastError());
         return AMSIM_OK;
@@ -809,7 +826,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         const int64_t nrows = row_end - split_seg->row_base;
         RArgs ra{ka.partial, d.out, nrows, d.J, split_seg->Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp,
                  split_seg->nsplit, d.batch, split_seg->row_base};
-        dim3 rgrid((unsigned)((nrows * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
+        dim3 rgrid((unsigned)((nrows * d.J + RED_OUTS - 1) / RED_OUTS), (unsigned)d.batch);
         splitk_reduce_kernel<<<rgrid, WG_THREADS, 0, stream>>>(ra);
         AMSIM_HIP_CHECK(hipGetLastError());
     }
