@@ -48,7 +48,6 @@ constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels ar
 constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
 constexpr int DEVICE_CUS = 256;               // MI355X; only steers work splitting, never correctness
 constexpr int WG_SLOTS = DEVICE_CUS * WAVES_PER_SIMD;  // workgroups resident at once
-constexpr int TARGET_WAVES = WG_SLOTS * 4;
 
 static std::atomic<int> g_split_k{1};
 
@@ -580,9 +579,11 @@ void lutgemm_kernel(KArgs a)
                 if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = acc[j];
         }
     } else {
-        float *o = a.partial + (((size_t)split * a.batch + bz) * seg_Rp + (r - seg_row_base)) * a.Jp + j0;
+        if (r < a.R) {  // rows past the end are never read by the reduction
+            float *o = a.partial + (((size_t)split * a.batch + bz) * seg_Rp + (r - seg_row_base)) * a.Jp + j0;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) o[j] = acc[j];
+            for (int j = 0; j < TN; ++j) o[j] = acc[j];
+        }
     }
 }
 
@@ -595,17 +596,18 @@ struct RArgs {
     int64_t row_base;
 };
 
-constexpr int RED_OUTS = 64;                      // outputs per workgroup
-constexpr int RED_WAYS = WG_THREADS / RED_OUTS;   // waves that share the splits of one output
-
-// Each wave takes every RED_WAYS-th split of 64 consecutive outputs in eight interleaved
-// chains (eight loads in flight); the chains and then the waves' sums are combined in a
-// fixed order, so the result does not depend on scheduling.
+// OUTS consecutive outputs per workgroup, WG_THREADS / OUTS threads ("ways") per output.  Each
+// way takes every ways-th split in eight interleaved chains (eight loads in flight); the chains
+// and then the ways' sums are combined in a fixed order, so the result does not depend on
+// scheduling.  Few outputs with many splits use OUTS = 8 (32 ways), else the loop over the
+// splits is one long chain of memory latencies.
+template <int OUTS>
 __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
 {
-    __shared__ float part[RED_WAYS][RED_OUTS];
-    const int o = threadIdx.x & (RED_OUTS - 1), way = threadIdx.x / RED_OUTS;
-    const int64_t idx = (int64_t)blockIdx.x * RED_OUTS + o;
+    constexpr int WAYS = WG_THREADS / OUTS;
+    __shared__ float part[WAYS][OUTS];
+    const int o = threadIdx.x % OUTS, way = threadIdx.x / OUTS;
+    const int64_t idx = (int64_t)blockIdx.x * OUTS + o;
     const int bz = blockIdx.y;
     const bool valid = idx < a.R * a.J;
     int64_t r = 0, j = 0;
@@ -616,20 +618,29 @@ __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
         const size_t stride = (size_t)a.batch * a.Rp * a.Jp;
         const float *src = a.partial + ((size_t)bz * a.Rp + r) * a.Jp + j;
         int sp = way;
-        for (; sp + 7 * RED_WAYS < a.nsplit; sp += 8 * RED_WAYS) {
+        for (; sp + 7 * WAYS < a.nsplit; sp += 8 * WAYS) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) c[u] += src[(size_t)(sp + u * RED_WAYS) * stride];
+            for (int u = 0; u < 8; ++u) c[u] += src[(size_t)(sp + u * WAYS) * stride];
         }
-        for (int u = 0; sp < a.nsplit; sp += RED_WAYS, ++u) c[u] += src[(size_t)sp * stride];
+        for (int u = 0; sp < a.nsplit; sp += WAYS, ++u) c[u] += src[(size_t)sp * stride];
     }
     part[way][o] = ((c[0] + c[1]) + (c[2] + c[3])) + ((c[4] + c[5]) + (c[6] + c[7]));
     __syncthreads();
     if (way == 0 && valid) {
         float s = part[0][o];
 #pragma unroll
-        for (int w = 1; w < RED_WAYS; ++w) s += part[w][o];
+        for (int w = 1; w < WAYS; ++w) s += part[w][o];
         a.out[(int64_t)bz * a.out_batch_stride + (a.row_base + r) * a.so_r + j * a.so_j] = s;
     }
+}
+
+static void launch_reduce(const RArgs &ra, hipStream_t stream)
+{
+    const int64_t outs = ra.R * ra.J;
+    if (outs * ra.batch <= 16384 && ra.nsplit >= 64)
+        splitk_reduce_kernel<8><<<dim3((unsigned)((outs + 7) / 8), (unsigned)ra.batch), WG_THREADS, 0, stream>>>(ra);
+    else
+        splitk_reduce_kernel<64><<<dim3((unsigned)((outs + 63) / 64), (unsigned)ra.batch), WG_THREADS, 0, stream>>>(ra);
 }
 
 // ---------------------------------------------------------------------------
@@ -653,17 +664,22 @@ static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 {
     Plan pl{};
-    pl.TN = J >= 9 ? 16 : J >= 5 ? 8 : J >= 3 ? 4 : (int)std::max<int64_t>(J, 1);
+    // Narrow outputs (one column group) stack four row tiles per workgroup and shrink the
+    // per-lane column count to fit; with a single row tile there is nothing to stack, and the
+    // 64-row kernel (compiled for 16 columns only) runs with its spare columns idle.
+    pl.TN = (J >= 9 || R <= 64) ? 16 : J >= 5 ? 8 : J >= 3 ? 4 : (int)std::max<int64_t>(J, 1);
     const int64_t jchunks = (J + pl.TN - 1) / pl.TN;
-    pl.WR = jchunks >= 2 ? 1 : 4;
+    pl.WR = (jchunks >= 2 || R <= 64) ? 1 : 4;
     pl.Jp = (int)((J + QT - 1) / QT * QT);
     pl.nchunks = (int)((K + KC - 1) / KC);
     const int rows = 64 * pl.WR;
     pl.Rp = (R + rows - 1) / rows * rows;
-    const int64_t waves = ((R + 63) / 64) * jchunks * batch;
+    const int64_t wgs = (pl.Rp / rows) * ((jchunks + 4 / pl.WR - 1) / (4 / pl.WR)) * batch;
+    const int64_t slots = pl.WR == 1 ? WG_SLOTS : DEVICE_CUS * 2;  // resident workgroups (the 256-row kernels run 2 per CU)
     pl.nsplit = 1;
-    if (g_split_k.load() && waves < TARGET_WAVES / 2 && pl.nchunks > 1) {
-        int64_t want = (TARGET_WAVES + waves - 1) / waves;
+    if (g_split_k.load() && wgs < slots / 2 && pl.nchunks > 1) {
+        // enough splits to fill the machine once
+        int64_t want = (slots + wgs - 1) / wgs;
         pl.nsplit = (int)std::min<int64_t>(want, pl.nchunks);
     }
     pl.chunks_per_split = (pl.nchunks + pl.nsplit - 1) / pl.nsplit;
@@ -675,8 +691,7 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
     if (g_split_k.load() && pl.nsplit == 1 && pl.WR == 1 && pl.nchunks >= 4) {
         const int64_t wgs_per_rowtile = ((jchunks + 3) / 4) * batch;
         const int64_t rowtiles = pl.Rp / rows;
-        const int64_t wgs = rowtiles * wgs_per_rowtile;
-        const int64_t full_rounds = wgs / WG_SLOTS;
+        const int64_t full_rounds = rowtiles * wgs_per_rowtile / WG_SLOTS;
         const int64_t main_tiles = full_rounds * WG_SLOTS / wgs_per_rowtile;
         const int64_t tail_wgs = (rowtiles - main_tiles) * wgs_per_rowtile;
         if (full_rounds >= 1 && tail_wgs > 0 && tail_wgs * 2 <= WG_SLOTS) {
@@ -752,8 +767,8 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
         RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0};
-        dim3 grid((unsigned)((d.R * d.J + RED_OUTS - 1) / RED_OUTS), (unsigned)d.batch);
-        splitk_reduce_kernel<<<grid, WG_THREADS, 0, stream>>>(ra);
+        if (d.batch > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
+        launch_reduce(ra, stream);
         AMSIM_HIP_CHECK(hipGetLastError());
         return AMSIM_OK;
     }
@@ -826,8 +841,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         const int64_t nrows = row_end - split_seg->row_base;
         RArgs ra{ka.partial, d.out, nrows, d.J, split_seg->Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp,
                  split_seg->nsplit, d.batch, split_seg->row_base};
-        dim3 rgrid((unsigned)((nrows * d.J + RED_OUTS - 1) / RED_OUTS), (unsigned)d.batch);
-        splitk_reduce_kernel<<<rgrid, WG_THREADS, 0, stream>>>(ra);
+        launch_reduce(ra, stream);
         AMSIM_HIP_CHECK(hipGetLastError());
     }
     return AMSIM_OK;
