@@ -185,17 +185,19 @@ int amsim_lut_load_file(const char *path, amsim_lut_t *out)
     int m = 0;
     int rc = parse_width_from_name(path, &m);
     if (rc != AMSIM_OK) return rc;
-    if (m < 1 || m > 7)
-        return fail(AMSIM_ERR_LUT_FORMAT, "LUT files hold one byte per entry: mantissa width must be 1..7, got " +
-                                              std::to_string(m));
+    if (m < 1 || m > 11)
+        return fail(AMSIM_ERR_LUT_FORMAT, "LUT file mantissa width must be 1..11, got " + std::to_string(m));
+    // one byte per entry up to width 7 (the reference's files); wider tables need more than
+    // 7 mantissa bits per entry and are stored in the 4-byte layout
+    const int entry_bytes = m <= 7 ? 1 : 4;
     std::ifstream file(path, std::ios::in | std::ios::binary);
     if (!file.is_open() || file.fail()) return fail(AMSIM_ERR_IO, std::string("lut file open failed: ") + path);
-    const size_t total = (size_t)1 << (2 * m);
+    const size_t total = ((size_t)1 << (2 * m)) * entry_bytes;
     std::vector<uint8_t> bytes(total);
     file.read(reinterpret_cast<char *>(bytes.data()), (std::streamsize)total);
     if ((size_t)file.gcount() != total)
         return fail(AMSIM_ERR_LUT_FORMAT, std::string("lut file too short: ") + path);
-    return amsim_lut_create(bytes.data(), total, m, 1, out);
+    return amsim_lut_create(bytes.data(), total, m, entry_bytes, out);
 }
 
 int amsim_lut_destroy(amsim_lut_t lut)

@@ -59,7 +59,9 @@ int amsim_device_info(char *arch, size_t arch_len, int *compute_units);
  *      (approx_mul_lut.h:7-80, cuda/approx_mul_lut.cu:24-53) -------------------
  * amsim_lut_load_file parses the mantissa width from the file name between the
  * last '_' and the last '.' (approx_mul_lut.h:22-25) and reads 2^(2m) entries:
- * 1 byte each (carry<<7 | mantissa, lut/lut_gen.cc:114-121) for m <= 7.
+ * 1 byte each (carry<<7 | mantissa, lut/lut_gen.cc:114-121) for m <= 7, 4 bytes
+ * each (the legacy layout below) for 8 <= m <= 11, which the reference has no
+ * file format for.
  * amsim_lut_create takes the entries from host memory; entry_bytes is 1
  * (layout above, m <= 7) or 4 (legacy layout of lut/AMsimulator.inl:18-20:
  * bit 31 = carry, bits 22..0 = mantissa in place; m <= 11). */
@@ -69,6 +71,24 @@ int amsim_lut_destroy(amsim_lut_t lut);
 int amsim_lut_mant_width(amsim_lut_t lut);
 /* the derived fields of approx_mul_lut.h:26-28 */
 int amsim_lut_params(amsim_lut_t lut, uint32_t *mant_mask, int *a_shift, int *b_shift);
+
+/* ---- LUT generation (host side): replaces lut/lut_gen.cc:86-127 + lut/lut_gen.sh
+ * A table holds, for every pair (i, j) of m-bit mantissas, the product of 1.i and
+ * 1.j at biased exponent 127: its top m mantissa bits and whether its exponent
+ * went up ("carry").  entry_bytes 1 (m <= 7): carry << 7 | mantissa, the file
+ * format of lut_gen.cc:114-121; entry_bytes 4 (m <= 11): carry << 31 | mantissa
+ * in place (lut/AMsimulator.inl:18-20).  `entries` is host memory of
+ * 2^(2m) * entry_bytes bytes; pass it to amsim_lut_create or write it to
+ * "<NAME>_<m>.bin" for amsim_lut_load_file (1-byte entries for m <= 7, 4-byte
+ * entries above).
+ * amsim_lut_generate evaluates a caller-supplied multiplier, the plug-in route
+ * of developer.md:38-86 (a C function taking and returning float);
+ * amsim_lut_generate_builtin knows "MBM" (lut/FPmultMBM_fast*.inl), "MIT"
+ * (lut/Mitchell_*.inl), "ACC" (lut/bfloat.inl at any width) and "ZEROS". */
+typedef float (*amsim_multiplier_fn)(float a, float b, void *user);
+int amsim_lut_generate(amsim_multiplier_fn fn, void *user, int mant_width, int entry_bytes, void *entries,
+                       size_t n_bytes);
+int amsim_lut_generate_builtin(const char *name, int mant_width, int entry_bytes, void *entries, size_t n_bytes);
 
 /* ---- elementwise product (test hook): the device function AMsimulator
  *      (cuda/AMsimulator.inl:13-36) with the functional models' semantics ---- */

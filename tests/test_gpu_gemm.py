@@ -219,3 +219,20 @@ def test_gemm_wide_mantissa_lut_gathered_from_global_memory(amd, kind, m):
         got = host(amd.gemm(lut, dev(A), dev(B), trans_a=bool(ta), trans_b=bool(tb)))
         want = cpu.gemm(img, m, A, B, transA=ta, transB=tb)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.gpu
+def test_generated_table_files_load_and_multiply(amd, tmp_path):
+    """Tables written by the generation tool (1-byte entries at width 5, 4-byte entries at
+    width 9) go through amsim_lut_load_file and give the oracle's GEMM bit for bit."""
+    from approxtrain_amd import ApproxMulLut, lut_gen
+    _set_split(0)
+    rng = np.random.default_rng(91)
+    for kind, m in (("MIT", 5), ("MBM", 9)):
+        entries = lut_gen.generate_builtin(kind, m, lut_gen.file_entry_bytes(m))
+        lut = ApproxMulLut(lut_gen.write_table(entries, kind, m, str(tmp_path)))
+        assert lut.mant_width == m
+        A, B = _ops(rng, 70, 40, 64, 0, 0)
+        got = host(amd.gemm(lut, dev(A), dev(B)))
+        want = cpu.gemm(cpu.lutgen32(kind, m), m, A, B)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

@@ -65,7 +65,8 @@ def test_lut_file_name_errors_do_not_exit(tmp_path):
     assert lib.amsim_lut_load_file(b"/nonexistent/MBM_7.bin", C.byref(h)) == 2          # I/O
     assert lib.amsim_lut_load_file(b"/nonexistent/nosuffix.bin", C.byref(h)) == 3       # no _<m>
     assert lib.amsim_lut_load_file(b"/nonexistent/MBM_x7.bin", C.byref(h)) == 3        # width not a number
-    assert lib.amsim_lut_load_file(b"/nonexistent/MBM_9.bin", C.byref(h)) == 3         # byte LUTs stop at m = 7
+    assert lib.amsim_lut_load_file(b"/nonexistent/MBM_12.bin", C.byref(h)) == 3        # widths stop at 11
+    assert lib.amsim_lut_load_file(b"/nonexistent/MBM_9.bin", C.byref(h)) == 2         # 8..11: 4-byte entries; I/O
     short = tmp_path / "MBM_7.bin"
     short.write_bytes(b"\x00" * 100)
     assert lib.amsim_lut_load_file(str(short).encode(), C.byref(h)) == 3               # short file
