@@ -420,17 +420,35 @@ void lutgemm_kernel(KArgs a)
             int y = (int)(t % a.p.GH);
             int b = (int)(t / a.p.GH);
             if (gf_uniform) {
-                // all rows of the tile share (fy, fx): the bounds test is wave-uniform and the
-                // address is a scalar pixel offset plus this lane's channel
+                // all rows of the tile share (fy, fx): the pixel walk, the window test and the
+                // pixel's source offset are wave-uniform and stay in scalar registers; a lane
+                // only adds its channel
+                x = __builtin_amdgcn_readfirstlane(x);
+                y = __builtin_amdgcn_readfirstlane(y);
+                b = __builtin_amdgcn_readfirstlane(b);
+                int iy = y * a.p.sy - a.p.pt + gf_fy, ix = x * a.p.sx - a.p.pl + gf_fx;
+                int soff = ((b * a.p.SH + iy) * a.p.SW + ix) * a.p.C + gf_c0;
+                const int step = a.p.sx * a.p.C;
+                const uint32_t chan = (uint32_t)rl;
+                const int64_t kleft64 = a.K - kfirst;
+                const int kleft = kleft64 < ELEMS ? (int)kleft64 : ELEMS;  // elements of this run inside K
 #pragma unroll
                 for (int i = 0; i < ELEMS; ++i) {
                     uint32_t v = 0;
-                    const int iy = y * a.p.sy - a.p.pt + gf_fy, ix = x * a.p.sx - a.p.pl + gf_fx;
-                    if (kfirst + i < a.K && (unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
-                        v = f2u(pbase[((b * a.p.SH + iy) * a.p.SW + ix) * a.p.C + gf_c0 + rl]);
+                    if (i < kleft && (unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
+                        v = f2u((pbase + soff)[chan]);
                     pv[i] = v;
                     sr.add(v);
-                    if (++x == a.p.GW) { x = 0; if (++y == a.p.GH) { y = 0; ++b; } }
+                    if (++x == a.p.GW) {
+                        x = 0;
+                        if (++y == a.p.GH) { y = 0; ++b; }
+                        iy = y * a.p.sy - a.p.pt + gf_fy;
+                        ix = gf_fx - a.p.pl;
+                        soff = ((b * a.p.SH + iy) * a.p.SW + ix) * a.p.C + gf_c0;
+                    } else {
+                        ix += a.p.sx;
+                        soff += step;
+                    }
                 }
             } else {
 #pragma unroll
