@@ -41,12 +41,14 @@ SIGNATURES = {
                             _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "amsim_convam_workspace_bytes": (_sz, [_i] * 7),
     "amsim_convam_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p, _sz, _p]),
+    "amsim_convam_bias_act_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _f, _i, _p, _sz, _p]),
     "amsim_convam_input_grad_workspace_bytes": (_sz, [_i] * 7),
     "amsim_convam_input_grad_f32": (_i, [_p, _f, _i, _i, _i, _i, _f] + [_i] * 9 + [_f, _i, _i, _p, _sz, _p]),
     "amsim_convam_filter_grad_workspace_bytes": (_sz, [_i] * 7),
     "amsim_convam_filter_grad_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p, _sz, _p]),
     "amsim_denseam_workspace_bytes": (_sz, [_i] * 3),
     "amsim_denseam_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),
+    "amsim_denseam_bias_act_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _f, _i, _p, _sz, _p]),
     "amsim_denseam_weight_grad_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),
     "amsim_denseam_input_grad_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),
     "amsim_matmulam_workspace_bytes": (_sz, [_i] * 6),

@@ -33,6 +33,8 @@ struct GemmCall {
     const float *B; int64_t ldb;
     float *C; int64_t ldc;
     int64_t batch, strideA, strideB, strideC;
+    const float *bias_n = nullptr;  // optional: added to C[.][n]
+    int act = AMSIM_ACT_NONE;
 };
 
 GemmDesc describe(const GemmCall &g)
@@ -50,6 +52,7 @@ GemmDesc describe(const GemmCall &g)
         d.q.batches = (g.batch > 1 && g.strideB != 0) ? (int)g.batch : 1;
         d.q.sk = g.transB ? 1 : g.ldb; d.q.sj = g.transB ? g.ldb : 1;
         d.so_r = g.ldc; d.so_j = 1;
+        d.bias_j = g.bias_n;
         d.lane_first = !g.swap;
     } else {
         d.R = g.N; d.J = g.M;
@@ -59,10 +62,14 @@ GemmDesc describe(const GemmCall &g)
         d.q.batches = (g.batch > 1 && g.strideA != 0) ? (int)g.batch : 1;
         d.q.sk = g.transA ? g.lda : 1; d.q.sj = g.transA ? 1 : g.lda;
         d.so_r = 1; d.so_j = g.ldc;
+        d.bias_r = g.bias_n;
         d.lane_first = g.swap != 0;
     }
+    d.act = g.act;
     return d;
 }
+
+bool known_activation(int act) { return act == AMSIM_ACT_NONE || act == AMSIM_ACT_RELU; }
 
 int gemm_call(amsim_lut_t lut, const GemmCall &g, void *ws, size_t ws_bytes, void *stream)
 {
@@ -133,6 +140,19 @@ int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_dat
                      int filter_top_offset, int filter_rows, int filter_cols, int in_depth, int input_cols,
                      int input_rows, const float *filter, void *workspace, size_t workspace_bytes, void *stream)
 {
+    return amsim_convam_bias_act_f32(lut, input_data, output_data, batch, out_rows, out_cols, out_depth, stride_cols,
+                                     stride_rows, filter_left_offset, filter_top_offset, filter_rows, filter_cols,
+                                     in_depth, input_cols, input_rows, filter, nullptr, AMSIM_ACT_NONE, workspace,
+                                     workspace_bytes, stream);
+}
+
+int amsim_convam_bias_act_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
+                              int out_cols, int out_depth, int stride_cols, int stride_rows,
+                              int filter_left_offset, int filter_top_offset, int filter_rows, int filter_cols,
+                              int in_depth, int input_cols, int input_rows, const float *filter, const float *bias,
+                              int activation, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!known_activation(activation)) return fail(AMSIM_ERR_INVALID, "unknown activation");
     if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
     if (batch < 0 || out_rows < 0 || out_cols < 0 || out_depth < 0 || filter_rows < 0 || filter_cols < 0 ||
         in_depth < 0 || input_cols < 0 || input_rows < 0 || stride_cols < 1 || stride_rows < 1)
@@ -152,6 +172,7 @@ int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_dat
     d.p.dy = 1; d.p.dx = 1; d.p.VH = input_rows; d.p.VW = input_cols; d.p.SH = input_rows; d.p.SW = input_cols;
     d.q.kind = Q_DENSE; d.q.base = filter; d.q.sk = out_depth; d.q.sj = 1;
     d.out = output_data; d.so_r = out_depth; d.so_j = 1;
+    d.bias_j = bias; d.act = activation;
     d.lane_first = true;  // P(input, filter)
     return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
@@ -254,6 +275,17 @@ int amsim_denseam_f32(amsim_lut_t lut, const float *inputs, const float *weights
 {
     // denseam_kernel.cu:38-41: P(input, weight)
     GemmCall g{0, 0, 0, batch, units, input_width, inputs, input_width, weights, units, output, units, 1, 0, 0, 0};
+    return gemm_call(lut, g, workspace, workspace_bytes, stream);
+}
+
+int amsim_denseam_bias_act_f32(amsim_lut_t lut, const float *inputs, const float *weights, float *output, int batch,
+                               int units, int input_width, const float *bias, int activation, void *workspace,
+                               size_t workspace_bytes, void *stream)
+{
+    if (!known_activation(activation)) return fail(AMSIM_ERR_INVALID, "unknown activation");
+    GemmCall g{0, 0, 0, batch, units, input_width, inputs, input_width, weights, units, output, units, 1, 0, 0, 0};
+    g.bias_n = bias;
+    g.act = activation;
     return gemm_call(lut, g, workspace, workspace_bytes, stream);
 }
 

@@ -59,6 +59,20 @@ enum { STAGE_R = 0,   // threads run along r, one element each (source contiguou
        STAGE_K = 1,   // threads run along k, one element each
        STAGE_K4 = 2 };// threads run along k, four consecutive k per 16-byte load
 
+// Output epilogue shared by the main kernel and the split reduction: bias add, then
+// the activation.  ReLU keeps NaN and the sign of a negative zero (x < 0 ? 0 : x).
+struct Epilogue {
+    const float *bias_j, *bias_r;
+    int act;
+};
+__device__ __forceinline__ float apply_epilogue(const Epilogue &e, float v, int64_t r, int64_t j)
+{
+    if (e.bias_j) v += e.bias_j[j];
+    if (e.bias_r) v += e.bias_r[r];
+    if (e.act == AMSIM_ACT_RELU) v = v < 0.0f ? 0.0f : v;
+    return v;
+}
+
 struct KArgs {
     PDesc p;
     const uint8_t *lut_img;  // LUT image indexed (uniform mantissa << m) | lane mantissa: bytes, or uint16 for m > 7
@@ -75,6 +89,7 @@ struct KArgs {
     int64_t so_r, so_j, out_batch_stride;
     float *partial;          // [nsplit][batch][Rp][Jp] of the segment whose nsplit > 1 (rows relative to its row_base)
     int batch;
+    Epilogue ep;
     // A launch covers up to two row segments, workgroups of seg[0] first in dispatch order:
     // seg[0] the split-reduction tail (if any), seg[1] the main part.
     struct Seg {
@@ -592,9 +607,15 @@ void lutgemm_kernel(KArgs a)
     if (seg_nsplit == 1) {
         if (r < a.R) {
             float *o = a.out + (int64_t)bz * a.out_batch_stride + r * a.so_r;
+            if (a.ep.bias_j || a.ep.bias_r || a.ep.act) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = acc[j];
+                for (int j = 0; j < TN; ++j)
+                    if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = apply_epilogue(a.ep, acc[j], r, j0 + j);
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = acc[j];
+            }
         }
     } else {
         if (r < a.R) {  // rows past the end are never read by the reduction
@@ -612,6 +633,7 @@ struct RArgs {
     int64_t R, J, Rp, so_r, so_j, out_batch_stride;  // R rows starting at row_base
     int Jp, nsplit, batch;
     int64_t row_base;
+    Epilogue ep;
 };
 
 // OUTS consecutive outputs per workgroup, WG_THREADS / OUTS threads ("ways") per output.  Each
@@ -648,7 +670,8 @@ __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
         float s = part[0][o];
 #pragma unroll
         for (int w = 1; w < WAYS; ++w) s += part[w][o];
-        a.out[(int64_t)bz * a.out_batch_stride + (a.row_base + r) * a.so_r + j * a.so_j] = s;
+        a.out[(int64_t)bz * a.out_batch_stride + (a.row_base + r) * a.so_r + j * a.so_j] =
+            apply_epilogue(a.ep, s, a.row_base + r, j);
     }
 }
 
@@ -784,7 +807,8 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         return fail(AMSIM_ERR_UNSUPPORTED, "LUT handle holds no device image for the GEMM path");
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
-        RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0};
+        RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0,
+                 Epilogue{d.bias_j, d.bias_r, d.act}};
         if (d.batch > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
         launch_reduce(ra, stream);
         AMSIM_HIP_CHECK(hipGetLastError());
@@ -822,6 +846,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.out = d.out; ka.so_r = d.so_r; ka.so_j = d.so_j; ka.out_batch_stride = d.out_batch_stride;
     ka.partial = reinterpret_cast<float *>(ws + pl.off_partial);
     ka.batch = d.batch;
+    ka.ep = Epilogue{d.bias_j, d.bias_r, d.act};
 
     const int rows = 64 * pl.WR, wc = 4 / pl.WR;
     const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;
@@ -858,7 +883,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         const int64_t row_end = split_seg == &ka.seg[0] ? d.R : pl.rows_main;
         const int64_t nrows = row_end - split_seg->row_base;
         RArgs ra{ka.partial, d.out, nrows, d.J, split_seg->Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp,
-                 split_seg->nsplit, d.batch, split_seg->row_base};
+                 split_seg->nsplit, d.batch, split_seg->row_base, ka.ep};
         launch_reduce(ra, stream);
         AMSIM_HIP_CHECK(hipGetLastError());
     }

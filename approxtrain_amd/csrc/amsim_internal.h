@@ -94,6 +94,10 @@ struct GemmDesc {
     float *out = nullptr;
     int64_t so_r = 0, so_j = 0, out_batch_stride = 0;
     bool lane_first = true;
+    // optional epilogue on every output element: + bias (indexed by j or by r, whichever
+    // dimension carries the output channels), then the activation
+    const float *bias_j = nullptr, *bias_r = nullptr;
+    int act = AMSIM_ACT_NONE;
 };
 
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches);

@@ -81,9 +81,27 @@ def gemm(lut, A, B, trans_a=False, trans_b=False, swap_operands=False):
     return out
 
 
-def convam(lut, input, filter, strides=(1, 1), padding="SAME"):
-    """ConvamFunctor: NHWC input, HWIO filter -> NHWC output."""
+ACTIVATIONS = {None: 0, "linear": 0, "relu": 1}
+
+
+def _epilogue(bias, activation, channels, device):
+    """Validates the optional fused epilogue; returns (bias tensor or None, bias pointer, activation code)."""
+    if activation not in ACTIVATIONS:
+        raise ValueError("fused activation must be None, 'linear' or 'relu'")
+    b = None
+    if bias is not None:
+        b = _dev(bias, "bias")
+        if b.dim() != 1 or b.shape[0] != channels:
+            raise ValueError("bias must have one entry per output channel")
+    return b, (_ptr(b) if b is not None else None), ACTIVATIONS[activation]
+
+
+def convam(lut, input, filter, strides=(1, 1), padding="SAME", bias=None, activation=None):
+    """ConvamFunctor: NHWC input, HWIO filter -> NHWC output.  With ``bias`` / ``activation``
+    the layer's BiasAdd and ReLU are applied as the result is stored (same values as the
+    separate ops)."""
     x, w = _dev(input, "input"), _dev(filter, "filter")
+    b, bptr, act = _epilogue(bias, activation, w.shape[3], x.device)
     lut = _lut(lut)
     n, h, wd, c = x.shape
     kh, kw, c2, oc = w.shape
@@ -95,8 +113,12 @@ def convam(lut, input, filter, strides=(1, 1), padding="SAME"):
     lib = load_library()
     nbytes = lib.amsim_convam_workspace_bytes(n, oh, ow, oc, kh, kw, c)
     ws, wsp = _workspace(nbytes, x.device)
-    check(lib.amsim_convam_f32(lut.handle, _ptr(x), _ptr(out), n, oh, ow, oc, strides[1], strides[0], pl, pt,
-                               kh, kw, c, wd, h, _ptr(w), wsp, nbytes, _stream()))
+    if b is None and act == 0:
+        check(lib.amsim_convam_f32(lut.handle, _ptr(x), _ptr(out), n, oh, ow, oc, strides[1], strides[0], pl, pt,
+                                   kh, kw, c, wd, h, _ptr(w), wsp, nbytes, _stream()))
+    else:
+        check(lib.amsim_convam_bias_act_f32(lut.handle, _ptr(x), _ptr(out), n, oh, ow, oc, strides[1], strides[0],
+                                            pl, pt, kh, kw, c, wd, h, _ptr(w), bptr, act, wsp, nbytes, _stream()))
     return out
 
 
@@ -147,15 +169,22 @@ def _dense_dims(x, w):
     return x.shape[0], w.shape[1], x.shape[1]
 
 
-def denseam(lut, inputs, weights):
+def denseam(lut, inputs, weights, bias=None, activation=None):
+    """DenseamFunctor; ``bias`` / ``activation`` fuse the layer's bias_add and ReLU into the store."""
     x, w = _dev(inputs, "inputs"), _dev(weights, "weights")
-    lut = _lut(lut)
     batch, units, width = _dense_dims(x, w)
+    b, bptr, act = _epilogue(bias, activation, units, x.device)
+    lut = _lut(lut)
     out = torch.empty((batch, units), dtype=torch.float32, device=x.device)
     lib = load_library()
     nbytes = lib.amsim_denseam_workspace_bytes(batch, units, width)
     ws, wsp = _workspace(nbytes, x.device)
-    check(lib.amsim_denseam_f32(lut.handle, _ptr(x), _ptr(w), _ptr(out), batch, units, width, wsp, nbytes, _stream()))
+    if b is None and act == 0:
+        check(lib.amsim_denseam_f32(lut.handle, _ptr(x), _ptr(w), _ptr(out), batch, units, width, wsp, nbytes,
+                                    _stream()))
+    else:
+        check(lib.amsim_denseam_bias_act_f32(lut.handle, _ptr(x), _ptr(w), _ptr(out), batch, units, width, bptr, act,
+                                             wsp, nbytes, _stream()))
     return out
 
 

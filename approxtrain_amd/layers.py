@@ -15,6 +15,49 @@ from .amnn_ops import amconvolution_v2
 from .math_ops import matmulam
 
 
+def _fusable(activation):
+    """Name of the activation if the library can apply it in the producing kernel, else None."""
+    if activation is None:
+        return "linear"
+    if activation in ("relu", torch.relu, torch.nn.functional.relu) or isinstance(activation, nn.ReLU):
+        return "relu"
+    return None
+
+
+def _epilogue_backward(grad, out, bias, act):
+    """Gradient through act(z + bias) given its output: (dL/dz, dL/dbias)."""
+    grad = grad.contiguous()
+    if act == "relu":
+        grad = grad * (out > 0)
+    grad_bias = grad.reshape(-1, grad.shape[-1]).sum(0) if bias is not None else None
+    return grad, grad_bias
+
+
+class _ConvamBiasAct(torch.autograd.Function):
+    """``act(Convam(input, filter) + bias)`` in one kernel (the reference runs Convam, BiasAdd
+    and the activation as three ops, am_convolutional.py:248-276); the gradient is the chain
+    rule through the epilogue followed by ConvamInputGrad / ConvamFilterGrad."""
+
+    @staticmethod
+    def forward(ctx, input, filters, bias, strides, padding, mant_mul_lut, act):
+        out = functors.convam(mant_mul_lut, input, filters, strides, padding, bias=bias, activation=act)
+        ctx.save_for_backward(input, filters, out)
+        ctx.attrs = (strides, padding, mant_mul_lut, act, bias is not None)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        input, filters, out = ctx.saved_tensors
+        strides, padding, lut, act, has_bias = ctx.attrs
+        grad, grad_bias = _epilogue_backward(grad, out, has_bias or None, act)
+        grad_input = grad_filter = None
+        if ctx.needs_input_grad[0]:
+            grad_input = functors.convam_input_grad(lut, input.shape, filters, grad, strides, padding)
+        if ctx.needs_input_grad[1]:
+            grad_filter = functors.convam_filter_grad(lut, input, filters.shape, grad, strides, padding)
+        return grad_input, grad_filter, grad_bias, None, None, None, None
+
+
 def _glorot_uniform_(t, fan_in, fan_out):
     limit = math.sqrt(6.0 / (fan_in + fan_out))
     with torch.no_grad():
@@ -57,6 +100,12 @@ class AMConv2D(nn.Module):
     def forward(self, inputs):
         if self.kernel is None:
             self.build(inputs.shape[-1], inputs.device)
+        act = _fusable(self.activation)
+        if act is not None and (self.use_bias or act != "linear"):
+            if inputs.dim() != 4 or inputs.shape[3] != self.kernel.shape[2]:
+                raise ValueError("input must be NHWC with the kernel's input depth")
+            return _ConvamBiasAct.apply(inputs, self.kernel, self.bias if self.use_bias else None,
+                                        tuple(self.strides), self.padding, self.mant_mul_lut, act)
         out = amconvolution_v2(inputs, self.kernel, strides=list(self.strides), padding=self.padding,
                                data_format="NHWC", mant_mul_lut=self.mant_mul_lut)
         if self.use_bias:
@@ -83,6 +132,26 @@ class _Denseam(torch.autograd.Function):
         inputs, weights = ctx.saved_tensors
         grad_input, grad_weights = functors.denseam_grad(ctx.lut, grad.contiguous(), inputs, weights)
         return grad_input, grad_weights, None
+
+
+class _DenseamBiasAct(torch.autograd.Function):
+    """``act(Denseam(inputs, weights) + bias)`` in one kernel (amdenselayer.py:211-226 runs
+    three ops); gradient = chain rule through the epilogue, then ``DenseamGrad``."""
+
+    @staticmethod
+    def forward(ctx, inputs, weights, bias, mant_mul_lut, act):
+        out = functors.denseam(mant_mul_lut, inputs, weights, bias=bias, activation=act)
+        ctx.save_for_backward(inputs, weights, out)
+        ctx.attrs = (mant_mul_lut, act, bias is not None)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        inputs, weights, out = ctx.saved_tensors
+        lut, act, has_bias = ctx.attrs
+        grad, grad_bias = _epilogue_backward(grad, out, has_bias or None, act)
+        grad_input, grad_weights = functors.denseam_grad(lut, grad, inputs, weights)
+        return grad_input, grad_weights, grad_bias, None, None
 
 
 class denseam(nn.Module):
@@ -112,7 +181,12 @@ class denseam(nn.Module):
         if self.kernel is None:
             self.build(inputs.shape[-1], inputs.device)
         lead = inputs.shape[:-1]
-        out = _Denseam.apply(inputs.reshape(-1, inputs.shape[-1]), self.kernel, self.mant_mul_lut)
+        flat = inputs.reshape(-1, inputs.shape[-1])
+        act = _fusable(self.activation)
+        if act is not None and (self.use_bias or act != "linear"):
+            out = _DenseamBiasAct.apply(flat, self.kernel, self.bias if self.use_bias else None, self.mant_mul_lut, act)
+            return out.reshape(tuple(lead) + (self.units,))
+        out = _Denseam.apply(flat, self.kernel, self.mant_mul_lut)
         out = out.reshape(tuple(lead) + (self.units,))
         if self.use_bias:
             out = out + self.bias

@@ -47,6 +47,10 @@ extern "C" {
 #define AMSIM_PADDING_VALID 1
 #define AMSIM_PADDING_SAME 2
 
+/* output epilogue of the *_bias_act entry points */
+#define AMSIM_ACT_NONE 0
+#define AMSIM_ACT_RELU 1
+
 typedef struct amsim_lut *amsim_lut_t;
 
 const char *amsim_status_string(int status);
@@ -119,6 +123,16 @@ int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_dat
                      int input_rows, const float *filter, void *workspace, size_t workspace_bytes,
                      void *stream);
 
+/* The same with the layer's epilogue fused into the store: output = act(conv + bias[out_depth]).
+ * Replaces Convam followed by BiasAdd and the activation op in AMConv2D.call
+ * (python/keras/layers/am_convolutional.py:248-276); bias may be NULL.  Bit-identical to the
+ * unfused sequence (the same FP32 add, then max with zero that keeps NaN). */
+int amsim_convam_bias_act_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
+                              int out_cols, int out_depth, int stride_cols, int stride_rows,
+                              int filter_left_offset, int filter_top_offset, int filter_rows, int filter_cols,
+                              int in_depth, int input_cols, int input_rows, const float *filter, const float *bias,
+                              int activation, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ConvamInputGradFunctor<GPUDevice,float>::operator() (convam.h:84-92,
  * cuda_kernel.cu:590-657).  pad_top/pad_left are the BACK pads
  * filter - 1 - forward_pad (convam.cc:1083-1084); hole_grad_* is the
@@ -146,6 +160,11 @@ size_t amsim_denseam_workspace_bytes(int batch, int units, int input_width);
 /* DenseamFunctor: output[batch][units] = inputs[batch][input_width] . weights[input_width][units] */
 int amsim_denseam_f32(amsim_lut_t lut, const float *inputs, const float *weights, float *output, int batch,
                       int units, int input_width, void *workspace, size_t workspace_bytes, void *stream);
+/* DenseamFunctor with the layer's epilogue fused: output = act(inputs . weights + bias[units])
+ * (amdenselayer.py:211-226: matmul, bias_add, activation); bias may be NULL. */
+int amsim_denseam_bias_act_f32(amsim_lut_t lut, const float *inputs, const float *weights, float *output, int batch,
+                               int units, int input_width, const float *bias, int activation, void *workspace,
+                               size_t workspace_bytes, void *stream);
 /* DenseamWeightGradFunctor: grad_weights[k][j] = sum_i P(input[i][k], grads[i][j]) */
 int amsim_denseam_weight_grad_f32(amsim_lut_t lut, const float *input, const float *grads, float *output,
                                   int batch, int units, int input_width, void *workspace,

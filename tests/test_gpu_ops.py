@@ -179,3 +179,79 @@ def test_multihead_attention_block_against_oracle_composition():
     # and it is differentiable end to end
     y.sum().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in mha.parameters())
+
+
+def _same_values(a, b):
+    """Equal element by element, NaN matching NaN (the sign of a zero is not compared)."""
+    a, b = host(a), host(b)
+    nan = np.isnan(a)
+    return np.array_equal(nan, np.isnan(b)) and np.array_equal(a[~nan], b[~nan])
+
+
+@pytest.mark.parametrize("split", [0, 1])
+@pytest.mark.parametrize("shape,filt,stride,padding", [((3, 9, 11, 8), (3, 3, 8, 20), 1, "SAME"),
+                                                        ((2, 12, 12, 4), (5, 5, 4, 3), 2, "VALID"),
+                                                        ((40, 14, 14, 32), (3, 3, 32, 64), 1, "SAME")])
+def test_fused_bias_relu_epilogue_equals_separate_ops(split, shape, filt, stride, padding):
+    """act(conv + bias) computed in the kernel's store (and in the split reduction when the
+    reduction is split) holds the same values as the three separate ops."""
+    import approxtrain_amd
+    from approxtrain_amd import functors
+    approxtrain_amd.load_library().amsim_set_split_k(split)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(*shape, device="cuda", generator=g)
+    w = torch.randn(*filt, device="cuda", generator=g)
+    b = torch.randn(filt[3], device="cuda", generator=g)
+    x[0, 1, 2, 0] = float("nan")
+    plain = functors.convam(MBM, x, w, (stride, stride), padding)
+    assert _same_values(functors.convam(MBM, x, w, (stride, stride), padding, bias=b), plain + b)
+    assert _same_values(functors.convam(MBM, x, w, (stride, stride), padding, activation="relu"), torch.relu(plain))
+    assert _same_values(functors.convam(MBM, x, w, (stride, stride), padding, bias=b, activation="relu"),
+                        torch.relu(plain + b))
+
+
+@pytest.mark.parametrize("batch,units,width", [(7, 10, 16), (300, 5, 64), (5, 300, 64), (128, 300, 784)])
+def test_fused_dense_epilogue_both_orientations(batch, units, width):
+    """The bias runs along the output's columns whichever GEMM dimension the kernel spreads over its lanes."""
+    from approxtrain_amd import functors
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x, w, b = (torch.randn(batch, width, device="cuda", generator=g), torch.randn(width, units, device="cuda", generator=g),
+               torch.randn(units, device="cuda", generator=g))
+    plain = functors.denseam(MBM, x, w)
+    assert _same_values(functors.denseam(MBM, x, w, bias=b, activation="relu"), torch.relu(plain + b))
+    assert _same_values(functors.denseam(MBM, x, w, bias=b), plain + b)
+
+
+def test_fused_epilogue_argument_errors():
+    from approxtrain_amd import functors
+    x, w = torch.zeros(1, 4, 4, 2, device="cuda"), torch.zeros(3, 3, 2, 5, device="cuda")
+    with pytest.raises(ValueError):
+        functors.convam(MBM, x, w, bias=torch.zeros(4, device="cuda"))
+    with pytest.raises(ValueError):
+        functors.convam(MBM, x, w, activation="tanh")
+
+
+def test_amconv2d_layer_fused_gradients_match_torch_on_integers():
+    """AMConv2D with bias and ReLU (one fused forward kernel): output, input / kernel / bias gradients
+    against float64 torch autograd, exact on small integers with the ACC_7 table."""
+    from approxtrain_amd.layers import AMConv2D
+    rng = np.random.default_rng(8)
+    layer = AMConv2D(5, 3, strides=(2, 2), padding="same", activation="relu", mant_mul_lut=ACC, in_channels=4).cuda()
+    w, b = small_ints(rng, (3, 3, 4, 5), -2, 2), small_ints(rng, (5,), -2, 2)
+    with torch.no_grad():
+        layer.kernel.copy_(dev(w)); layer.bias.copy_(dev(b))
+    x = small_ints(rng, (2, 9, 7, 4), -2, 2)
+    xt = dev(x).requires_grad_(True)
+    y = layer(xt)
+    gy = small_ints(rng, tuple(y.shape), -2, 2)
+    y.backward(dev(gy))
+    x64 = torch.tensor(x, dtype=torch.float64).permute(0, 3, 1, 2).requires_grad_(True)
+    w64 = torch.tensor(w, dtype=torch.float64).permute(3, 2, 0, 1).requires_grad_(True)
+    b64 = torch.tensor(b, dtype=torch.float64, requires_grad=True)
+    # SAME with stride 2 on 9 x 7: output 5 x 4, total padding (2, 2) -> 1 before, 1 after
+    ref = torch.relu(torch.nn.functional.conv2d(torch.nn.functional.pad(x64, (1, 1, 1, 1)), w64, b64, stride=2))
+    ref.backward(torch.tensor(gy, dtype=torch.float64).permute(0, 3, 1, 2))
+    assert np.array_equal(host(y).astype(np.float64), ref.detach().permute(0, 2, 3, 1).numpy())
+    assert np.array_equal(host(xt.grad).astype(np.float64), x64.grad.permute(0, 2, 3, 1).numpy())
+    assert np.array_equal(host(layer.kernel.grad).astype(np.float64), w64.grad.permute(2, 3, 1, 0).numpy())
+    assert np.array_equal(host(layer.bias.grad).astype(np.float64), b64.grad.numpy())
