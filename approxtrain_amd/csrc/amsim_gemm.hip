@@ -87,13 +87,13 @@ struct KArgs {
     int Jp, nchunks;
     float *out;
     int64_t so_r, so_j, out_batch_stride;
-    float *partial;          // [nsplit][batch][Rp][Jp] of the segment whose nsplit > 1 (rows relative to its row_base)
     int batch;
     Epilogue ep;
     // A launch covers up to two row segments, workgroups of seg[0] first in dispatch order:
     // seg[0] the split-reduction tail (if any), seg[1] the main part.
     struct Seg {
         int64_t row_base, Rp;        // first row, padded row count
+        float *partial;              // [nsplit][batch][Rp][Jp] when nsplit > 1 (rows relative to row_base)
         int nsplit, chunks_per_split;
         unsigned X, Y, Z;            // row tiles, column groups, batch x splits
         unsigned total;              // X * Y * Z
@@ -229,6 +229,7 @@ void lutgemm_kernel(KArgs a)
     const bool in_first = blockIdx.x < a.seg[0].total;
     const int64_t seg_row_base = in_first ? a.seg[0].row_base : a.seg[1].row_base;
     const int64_t seg_Rp = in_first ? a.seg[0].Rp : a.seg[1].Rp;
+    float *const seg_partial = in_first ? a.seg[0].partial : a.seg[1].partial;
     const int seg_nsplit = in_first ? a.seg[0].nsplit : a.seg[1].nsplit;
     const int seg_cps = in_first ? a.seg[0].chunks_per_split : a.seg[1].chunks_per_split;
     unsigned bx, by, bzz;
@@ -619,7 +620,7 @@ void lutgemm_kernel(KArgs a)
         }
     } else {
         if (r < a.R) {  // rows past the end are never read by the reduction
-            float *o = a.partial + (((size_t)split * a.batch + bz) * seg_Rp + (r - seg_row_base)) * a.Jp + j0;
+            float *o = seg_partial + (((size_t)split * a.batch + bz) * seg_Rp + (r - seg_row_base)) * a.Jp + j0;
 #pragma unroll
             for (int j = 0; j < TN; ++j) o[j] = acc[j];
         }
@@ -687,22 +688,111 @@ static void launch_reduce(const RArgs &ra, hipStream_t stream)
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-// A call is one launch, or two when the workgroup count is a little more than a
-// whole number of machine-filling rounds: the rows of the last, mostly empty
-// round ("tail") are then launched separately with the reduction split across
-// enough workgroups to fill the machine again.
+// Work shaping.  A problem is R/rows row tiles x column groups x batch workgroups ("tiles"),
+// each a reduction of nchunks chunks.  The machine holds `slots` workgroups at once and a
+// lone workgroup runs about 1/0.74 as fast as one of a full machine, so the time of a launch
+// is governed by rounds of `slots` workgroups.  The planner picks
+//   * nsplit: every tile's reduction split into that many workgroups (partial sums reduced by
+//     splitk_reduce_kernel in a fixed order), and
+//   * a tail: when the workgroup count is a little more than a whole number of rounds, the
+//     row tiles of the last, mostly empty round are split further so that they fill the
+//     machine again (their workgroups dispatch first, in the same launch),
+// by minimising a small cost model (unit: one chunk of one workgroup on a full machine).
 struct Plan {
     int TN, WR, Jp, nchunks;
-    int nsplit, chunks_per_split;  // of the main launch
-    int64_t Rp;                    // padded rows of the launch that writes partials
-    int64_t rows_main;             // rows covered by the main launch (== R when there is no tail)
+    int nsplit, chunks_per_split;  // of the main part
+    int64_t Rp;                    // padded rows
+    int64_t rows_main;             // rows covered by the main part (== R when there is no tail)
     int tail_nsplit, tail_chunks_per_split;
-    size_t off_qw, off_qraw, off_flags, off_partial, total;
+    size_t off_qw, off_qraw, off_flags, off_partial_main, off_partial_tail, total;
 };
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
+namespace {
+struct Shape {
+    int nsplit = 1, cps = 0;
+    int64_t main_rowtiles = 0;
+    int tail_nsplit = 1, tail_cps = 0;
+    double cost = 0;
+};
+// Time of one chunk of one workgroup when a fraction `occ` of the machine's workgroup slots is
+// filled, relative to a full machine (measured: 0.735 at 51 %; nearly linear above that).
+inline double occupancy_factor(double occ)
+{
+    if (occ >= 1.0) return 1.0;
+    return occ >= 0.51 ? 0.735 + 0.54 * (occ - 0.51) : 0.735 - 0.5 * (0.51 - occ);
+}
+}  // namespace
+
+static Shape shape_work(int64_t rowtiles, int64_t G, int n, int64_t slots, bool may_peel, double reduce_unit)
+{
+    // reduce_unit: cost of writing + re-reading one full set of partial sums
+    Shape best;
+    best.cps = n;
+    best.main_rowtiles = rowtiles;
+    best.tail_cps = n;
+    bool have = false;
+    const int64_t wgs = rowtiles * G;
+    const int64_t smax = std::min<int64_t>(n, 2 * ((slots + wgs - 1) / wgs) + 1);
+    for (int64_t s0 = 1; s0 <= smax; ++s0) {
+        Shape c;
+        c.cps = (int)((n + s0 - 1) / s0);
+        c.nsplit = (n + c.cps - 1) / c.cps;
+        if (c.nsplit != s0) continue;  // same shape as a smaller candidate
+        c.main_rowtiles = rowtiles;
+        c.tail_cps = n;
+        const int64_t units = wgs * c.nsplit;
+        const int64_t full = units / slots, rem = units - full * slots;
+        double t;
+        if (full == 0) {
+            t = c.cps * occupancy_factor((double)units / slots);
+        } else if (rem == 0) {
+            t = (double)full * c.cps;
+        } else {
+            t = (double)full * c.cps + c.cps * occupancy_factor((double)rem / slots);
+            const int64_t main_rt = full * slots / (G * c.nsplit);
+            const int64_t tail_wgs = (rowtiles - main_rt) * G;
+            if (may_peel && main_rt >= 1 && tail_wgs * c.nsplit * 2 <= slots) {
+                const int64_t ts0 = std::min<int64_t>(slots / tail_wgs, n);
+                const int tcps = (int)((n + ts0 - 1) / ts0);
+                const int ts = (n + tcps - 1) / tcps;
+                if (ts > c.nsplit) {
+                    const double tp = (double)full * c.cps + tcps * occupancy_factor((double)tail_wgs * ts / slots) + 0.8;
+                    if (tp < t) { t = tp; c.main_rowtiles = main_rt; c.tail_nsplit = ts; c.tail_cps = tcps; }
+                }
+            }
+        }
+        if (c.nsplit > 1) t += 0.4 + reduce_unit * c.nsplit;
+        c.cost = t;
+        if (!have || t < best.cost - 1e-9) { best = c; have = true; }
+    }
+    return best;
+}
+
+static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k);
+
+// Plans are pure functions of their arguments; the last few are remembered per thread so that
+// the workspace query and the call that follows it do not repeat the search.
+static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k)
+{
+    struct Key { int64_t R, J, K; int batch, qb, split; };
+    struct Slot { Key k; Plan p; bool used = false; };
+    static thread_local Slot memo[8];
+    static thread_local unsigned next = 0;
+    const Key key{R, J, K, batch, q_batches, split_k ? 1 : 0};
+    for (const Slot &sl : memo)
+        if (sl.used && sl.k.R == R && sl.k.J == J && sl.k.K == K && sl.k.batch == batch && sl.k.qb == q_batches &&
+            sl.k.split == key.split)
+            return sl.p;
+    Slot &sl = memo[next++ % 8];
+    sl.k = key;
+    sl.p = compute_plan(R, J, K, batch, q_batches, split_k);
+    sl.used = true;
+    return sl.p;
+}
+
+static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k)
 {
     Plan pl{};
     // Narrow outputs (one column group) stack four row tiles per workgroup and shrink the
@@ -713,46 +803,39 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
     pl.WR = (jchunks >= 2 || R <= 64) ? 1 : 4;
     pl.Jp = (int)((J + QT - 1) / QT * QT);
     pl.nchunks = (int)((K + KC - 1) / KC);
-    const int rows = 64 * pl.WR;
+    const int rows = 64 * pl.WR, wc = 4 / pl.WR;
     pl.Rp = (R + rows - 1) / rows * rows;
-    const int64_t wgs = (pl.Rp / rows) * ((jchunks + 4 / pl.WR - 1) / (4 / pl.WR)) * batch;
+    const int64_t rowtiles = pl.Rp / rows;
+    const int64_t G = ((jchunks + wc - 1) / wc) * batch;
     const int64_t slots = pl.WR == 1 ? WG_SLOTS : DEVICE_CUS * 2;  // resident workgroups (the 256-row kernels run 2 per CU)
-    pl.nsplit = 1;
-    if (g_split_k.load() && wgs < slots / 2 && pl.nchunks > 1) {
-        // enough splits to fill the machine once
-        int64_t want = (slots + wgs - 1) / wgs;
-        pl.nsplit = (int)std::min<int64_t>(want, pl.nchunks);
+
+    Shape sh;
+    sh.cps = pl.nchunks;
+    sh.main_rowtiles = rowtiles;
+    sh.tail_cps = pl.nchunks;
+    if (split_k && pl.nchunks > 1) {
+        // one chunk of one workgroup on a full machine, and one pass over the output, in seconds
+        const double chunk_s = (double)rows * (wc * pl.TN) * KC * slots / 13.0e12;
+        const double pass_s = 2.0 * (double)pl.Rp * pl.Jp * batch * sizeof(float) / 3.0e12;
+        sh = shape_work(rowtiles, G, pl.nchunks, slots, pl.WR == 1, pass_s / chunk_s);
     }
-    pl.chunks_per_split = (pl.nchunks + pl.nsplit - 1) / pl.nsplit;
-    pl.nsplit = (pl.nchunks + pl.chunks_per_split - 1) / std::max(pl.chunks_per_split, 1);
-    if (pl.nchunks == 0) { pl.nsplit = 1; pl.chunks_per_split = 0; }
-    pl.rows_main = R;
-    pl.tail_nsplit = 1;
-    pl.tail_chunks_per_split = pl.nchunks;
-    if (g_split_k.load() && pl.nsplit == 1 && pl.WR == 1 && pl.nchunks >= 4) {
-        const int64_t wgs_per_rowtile = ((jchunks + 3) / 4) * batch;
-        const int64_t rowtiles = pl.Rp / rows;
-        const int64_t full_rounds = rowtiles * wgs_per_rowtile / WG_SLOTS;
-        const int64_t main_tiles = full_rounds * WG_SLOTS / wgs_per_rowtile;
-        const int64_t tail_wgs = (rowtiles - main_tiles) * wgs_per_rowtile;
-        if (full_rounds >= 1 && tail_wgs > 0 && tail_wgs * 2 <= WG_SLOTS) {
-            int ts = (int)std::min<int64_t>(WG_SLOTS / tail_wgs, pl.nchunks);
-            if (ts >= 2) {
-                pl.rows_main = main_tiles * rows;
-                pl.tail_chunks_per_split = (pl.nchunks + ts - 1) / ts;
-                pl.tail_nsplit = (pl.nchunks + pl.tail_chunks_per_split - 1) / pl.tail_chunks_per_split;
-            }
-        }
-    }
+    pl.nsplit = sh.nsplit;
+    pl.chunks_per_split = sh.cps;
+    pl.rows_main = sh.main_rowtiles == rowtiles ? R : sh.main_rowtiles * rows;
+    pl.tail_nsplit = sh.tail_nsplit;
+    pl.tail_chunks_per_split = sh.tail_cps;
+
     const size_t plane = (size_t)pl.nchunks * KC * pl.Jp;
     size_t off = 0;
     pl.off_qw = off;      off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
     pl.off_qraw = off;    off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
     pl.off_flags = off;   off = align256(off + (size_t)q_batches * (pl.Jp / QT) * std::max(pl.nchunks, 1) * sizeof(uint32_t));
-    pl.off_partial = off;
-    if (pl.nsplit > 1) off = align256(off + (size_t)pl.nsplit * batch * pl.Rp * pl.Jp * sizeof(float));
-    else if (pl.tail_nsplit > 1)
-        off = align256(off + (size_t)pl.tail_nsplit * batch * (pl.Rp - pl.rows_main) * pl.Jp * sizeof(float));
+    const int64_t main_rows_p = sh.main_rowtiles * rows, tail_rows_p = pl.Rp - main_rows_p;
+    pl.off_partial_main = off;
+    if (pl.nsplit > 1) off = align256(off + (size_t)pl.nsplit * batch * main_rows_p * pl.Jp * sizeof(float));
+    pl.off_partial_tail = off;
+    if (pl.rows_main < R && pl.tail_nsplit > 1)
+        off = align256(off + (size_t)pl.tail_nsplit * batch * tail_rows_p * pl.Jp * sizeof(float));
     pl.total = off;
     return pl;
 }
@@ -760,7 +843,8 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 {
     if (R <= 0 || J <= 0 || K <= 0 || batch <= 0) return 0;
-    return make_plan(R, J, K, batch, q_batches).total;
+    // valid whichever way amsim_set_split_k stands when the call is made
+    return std::max(make_plan(R, J, K, batch, q_batches, true).total, make_plan(R, J, K, batch, q_batches, false).total);
 }
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -816,10 +900,12 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     }
     if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
-    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches);
-    if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < pl.total)
+    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, g_split_k.load() != 0);
+    // the size the query returns (valid for either split mode), not just this plan's
+    const size_t need = gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
+    if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need)
         return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
-                                             std::to_string(pl.total) + " bytes");
+                                             std::to_string(need) + " bytes");
     uint8_t *ws = static_cast<uint8_t *>(workspace);
 
     QArgs qa{};
@@ -844,7 +930,6 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.R = d.R; ka.J = d.J; ka.K = d.K;
     ka.Jp = pl.Jp; ka.nchunks = pl.nchunks;
     ka.out = d.out; ka.so_r = d.so_r; ka.so_j = d.so_j; ka.out_batch_stride = d.out_batch_stride;
-    ka.partial = reinterpret_cast<float *>(ws + pl.off_partial);
     ka.batch = d.batch;
     ka.ep = Epilogue{d.bias_j, d.bias_r, d.act};
 
@@ -855,8 +940,9 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     // One launch: the split-reduction tail's workgroups (if any) come first in dispatch order
     // and share the machine with the first main workgroups; the main workgroups that start
     // after them catch up through wave priority.
-    auto fill_seg = [&](KArgs::Seg &sg, int64_t row_base, int64_t row_end, int nsplit, int cps) -> int64_t {
+    auto fill_seg = [&](KArgs::Seg &sg, int64_t row_base, int64_t row_end, int nsplit, int cps, size_t off_partial) -> int64_t {
         sg.row_base = row_base;
+        sg.partial = reinterpret_cast<float *>(ws + off_partial);
         sg.Rp = (row_end - row_base + rows - 1) / rows * rows;
         sg.nsplit = nsplit;
         sg.chunks_per_split = cps;
@@ -868,22 +954,22 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     };
     const bool has_tail = pl.rows_main < d.R;
     int64_t total = 0;
-    if (has_tail) total += fill_seg(ka.seg[0], pl.rows_main, d.R, pl.tail_nsplit, pl.tail_chunks_per_split);
-    else ka.seg[0] = KArgs::Seg{0, 0, 1, 0, 0, 0, 0, 0};
-    total += fill_seg(ka.seg[1], 0, pl.rows_main, pl.nsplit, pl.chunks_per_split);
+    if (has_tail) total += fill_seg(ka.seg[0], pl.rows_main, d.R, pl.tail_nsplit, pl.tail_chunks_per_split, pl.off_partial_tail);
+    else ka.seg[0] = KArgs::Seg{0, 0, nullptr, 1, 0, 0, 0, 0, 0};
+    total += fill_seg(ka.seg[1], 0, pl.rows_main, pl.nsplit, pl.chunks_per_split, pl.off_partial_main);
     if (total >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "workgroup count exceeds the grid limit");
     const dim3 grid((unsigned)total);
     if (lut.m > 7) launch_tn<true>(pl.TN, pl.WR, ka, grid, stream);
     else launch_tn<false>(pl.TN, pl.WR, ka, grid, stream);
     AMSIM_HIP_CHECK(hipGetLastError());
 
-    const KArgs::Seg *split_seg = has_tail && pl.tail_nsplit > 1 ? &ka.seg[0] : pl.nsplit > 1 ? &ka.seg[1] : nullptr;
-    if (split_seg) {
+    for (int sgi = 0; sgi < 2; ++sgi) {
+        const KArgs::Seg &sg = ka.seg[sgi];
+        if (sg.total == 0 || sg.nsplit <= 1) continue;
         if (d.batch > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
-        const int64_t row_end = split_seg == &ka.seg[0] ? d.R : pl.rows_main;
-        const int64_t nrows = row_end - split_seg->row_base;
-        RArgs ra{ka.partial, d.out, nrows, d.J, split_seg->Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp,
-                 split_seg->nsplit, d.batch, split_seg->row_base, ka.ep};
+        const int64_t row_end = sgi == 0 ? d.R : pl.rows_main;
+        RArgs ra{sg.partial, d.out, row_end - sg.row_base, d.J, sg.Rp, d.so_r, d.so_j, d.out_batch_stride, pl.Jp,
+                 sg.nsplit, d.batch, sg.row_base, ka.ep};
         launch_reduce(ra, stream);
         AMSIM_HIP_CHECK(hipGetLastError());
     }
