@@ -4,6 +4,7 @@
 #include "amsim_internal.h"
 
 #include <algorithm>
+#include <string>
 
 namespace amsim {
 void set_split_k(int mode);
@@ -177,11 +178,88 @@ int amsim_convam_bias_act_f32(amsim_lut_t lut, const float *input_data, float *o
     return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+// ---- grad-input ----------------------------------------------------------------------
+// The reference dilates the gradient with (stride - 1) zeros between samples and multiplies
+// every filter tap with it (cuda_kernel.cu:463-502, 569-583).  Input pixels whose row / column
+// index has the same residue modulo the stride meet the same subset of taps (the others hit the
+// inserted zeros, whose products are +0 and leave the FP32 sum unchanged), so the problem is
+// run as stride_rows x stride_cols undilated sub-problems ("phases"), each over its own pixels
+// and taps, in the reference's reduction order.  Stride 1 is the single phase (0, 0).
+namespace {
+
+struct Phase {
+    int n_out;   // input pixels along this axis in the phase
+    int taps;    // filter taps that meet gradient samples
+    int f0;      // first such tap (index into the flipped filter)
+    int pad;     // leading pad of the undilated patch: source = pixel - pad + tap
+};
+
+Phase phase_of(int extent, int stride, int residue, int filter, int back_pad)
+{
+    Phase ph;
+    ph.n_out = residue < extent ? (extent - residue + stride - 1) / stride : 0;
+    ph.f0 = ((back_pad - residue) % stride + stride) % stride;
+    ph.taps = ph.f0 < filter ? (filter - ph.f0 + stride - 1) / stride : 0;
+    ph.pad = -((residue - back_pad + ph.f0) / stride);  // exact: the numerator is a multiple of the stride
+    return ph;
+}
+
+struct GradInputGeometry {
+    int batch, input_rows, input_cols, in_depth, filter_rows, filter_cols, out_depth, out_rows, out_cols;
+    int stride_rows, stride_cols, pad_top, pad_left;
+};
+
+GemmDesc grad_input_phase(const GradInputGeometry &g, int py, int px, const float *grad, const float *filter,
+                          float *output)
+{
+    const Phase y = phase_of(g.input_rows, g.stride_rows, py, g.filter_rows, g.pad_top);
+    const Phase x = phase_of(g.input_cols, g.stride_cols, px, g.filter_cols, g.pad_left);
+    GemmDesc d;
+    d.R = (int64_t)g.batch * y.n_out * x.n_out;
+    d.J = g.in_depth;
+    d.K = (int64_t)y.taps * x.taps * g.out_depth;
+    d.p.kind = P_PATCH; d.p.base = grad;
+    d.p.B = g.batch; d.p.GH = y.n_out; d.p.GW = x.n_out;
+    d.p.KH = y.taps; d.p.KW = x.taps; d.p.C = g.out_depth;
+    d.p.sy = 1; d.p.sx = 1; d.p.pt = y.pad; d.p.pl = x.pad;
+    d.p.dy = 1; d.p.dx = 1; d.p.VH = g.out_rows; d.p.VW = g.out_cols; d.p.SH = g.out_rows; d.p.SW = g.out_cols;
+    d.q.kind = Q_FLIP; d.q.base = filter;
+    d.q.KH = g.filter_rows; d.q.KW = g.filter_cols; d.q.IC = g.in_depth; d.q.OC = g.out_depth;
+    d.q.TH = y.taps; d.q.TW = x.taps; d.q.fy0 = y.f0; d.q.fx0 = x.f0; d.q.fsy = g.stride_rows; d.q.fsx = g.stride_cols;
+    d.out = output; d.so_r = g.in_depth; d.so_j = 1;
+    d.omap.enabled = (g.stride_rows > 1 || g.stride_cols > 1) ? 1 : 0;
+    d.omap.GH = y.n_out; d.omap.GW = x.n_out; d.omap.sy = g.stride_rows; d.omap.sx = g.stride_cols;
+    d.omap.oy = py; d.omap.ox = px; d.omap.H = g.input_rows; d.omap.W = g.input_cols;
+    d.lane_first = true;  // P(grad, filter)
+    return d;
+}
+
+}  // namespace
+
 size_t amsim_convam_input_grad_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
                                                int filter_rows, int filter_cols, int out_depth)
 {
+    // The strides are not part of the query (as they are not part of the reference's temporaries'
+    // shapes): a strided call runs smaller sub-problems than this stride-1 bound in every extent.
     return gemm_workspace_bytes((int64_t)batch * input_rows * input_cols, in_depth,
                                 (int64_t)filter_rows * filter_cols * out_depth, 1, 1);
+}
+
+size_t amsim_convam_input_grad_strided_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
+                                                       int filter_rows, int filter_cols, int out_depth,
+                                                       int stride_rows, int stride_cols, int pad_top, int pad_left)
+{
+    size_t need = amsim_convam_input_grad_workspace_bytes(batch, input_rows, input_cols, in_depth, filter_rows,
+                                                          filter_cols, out_depth);
+    if (stride_rows < 1 || stride_cols < 1 || batch <= 0 || input_rows <= 0 || input_cols <= 0) return need;
+    const GradInputGeometry g{batch, input_rows, input_cols, in_depth, filter_rows, filter_cols, out_depth,
+                              0, 0, stride_rows, stride_cols, pad_top, pad_left};
+    for (int py = 0; py < stride_rows; ++py)
+        for (int px = 0; px < stride_cols; ++px) {
+            const GemmDesc d = grad_input_phase(g, py, px, nullptr, nullptr, nullptr);
+            need = std::max(need, gemm_workspace_bytes(d.R, d.J, d.K, 1, 1));
+        }
+    return need;
 }
 
 int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_grad_width, int hole_grad_height,
@@ -202,22 +280,25 @@ int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_gra
     if (!grad || !output || !filter) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
     if (!fits_int32((int64_t)batch * out_rows * out_cols * out_depth))
         return fail(AMSIM_ERR_UNSUPPORTED, "gradient tensor has 2^31 or more elements");
-    // rows (b, y, x) of the input x columns (fy, fx, oc) of the zero-dilated,
-    // back-padded gradient [cuda_kernel.cu:463-502]; the flipped, I/O-swapped
-    // filter [reverseNswapdim23.cu:16] is produced by the operand pre-pass.
-    GemmDesc d;
-    d.R = R; d.J = in_depth; d.K = (int64_t)filter_rows * filter_cols * out_depth;
-    d.p.kind = P_PATCH; d.p.base = grad;
-    d.p.B = batch; d.p.GH = input_rows; d.p.GW = input_cols;
-    d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = out_depth;
-    d.p.sy = 1; d.p.sx = 1; d.p.pt = pad_top; d.p.pl = pad_left;
-    d.p.dy = stride_rows; d.p.dx = stride_cols; d.p.VH = hole_grad_height; d.p.VW = hole_grad_width;
-    d.p.SH = out_rows; d.p.SW = out_cols;
-    d.q.kind = Q_FLIP; d.q.base = filter; d.q.KH = filter_rows; d.q.KW = filter_cols; d.q.IC = in_depth;
-    d.q.OC = out_depth;
-    d.out = output; d.so_r = in_depth; d.so_j = 1;
-    d.lane_first = true;  // P(grad, filter)
-    return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    if (!fits_int32(R * in_depth)) return fail(AMSIM_ERR_UNSUPPORTED, "input tensor has 2^31 or more elements");
+    const size_t need = amsim_convam_input_grad_workspace_bytes(batch, input_rows, input_cols, in_depth, filter_rows,
+                                                                filter_cols, out_depth);
+    if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need)
+        return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
+                                             std::to_string(need) + " bytes");
+    const GradInputGeometry g{batch, input_rows, input_cols, in_depth, filter_rows, filter_cols, out_depth,
+                              out_rows, out_cols, stride_rows, stride_cols, pad_top, pad_left};
+    for (int py = 0; py < stride_rows; ++py)
+        for (int px = 0; px < stride_cols; ++px) {
+            GemmDesc d = grad_input_phase(g, py, px, grad, filter, output);
+            if (d.R == 0) continue;
+            // a phase whose best plan wants more partial-sum space than the caller's (stride-agnostic)
+            // workspace holds runs unsplit: its pre-decoded filter always fits
+            if (gemm_workspace_bytes(d.R, d.J, d.K, 1, 1) > workspace_bytes) d.no_split = true;
+            const int rc = run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+            if (rc != AMSIM_OK) return rc;
+        }
+    return AMSIM_OK;
 }
 
 size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth,

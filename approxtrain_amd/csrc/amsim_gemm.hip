@@ -64,7 +64,18 @@ enum { STAGE_R = 0,   // threads run along r, one element each (source contiguou
 struct Epilogue {
     const float *bias_j, *bias_r;
     int act;
+    OutMap omap;
 };
+// element offset of output row r (before the column term)
+__device__ __forceinline__ int64_t out_row_offset(const OutMap &m, int64_t r, int64_t so_r)
+{
+    if (!m.enabled) return r * so_r;
+    const int x = (int)(r % m.GW);
+    const int64_t t = r / m.GW;
+    const int y = (int)(t % m.GH);
+    const int64_t b = t / m.GH;
+    return ((b * m.H + (y * m.sy + m.oy)) * m.W + (x * m.sx + m.ox)) * so_r;
+}
 __device__ __forceinline__ float apply_epilogue(const Epilogue &e, float v, int64_t r, int64_t j)
 {
     if (e.bias_j) v += e.bias_j[j];
@@ -145,7 +156,7 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
             } else {
                 const int oc = (int)(k % a.q.OC);
                 const int t = (int)(k / a.q.OC);
-                const int fx = t % a.q.KW, fy = t / a.q.KW;
+                const int fx = a.q.fx0 + (t % a.q.TW) * a.q.fsx, fy = a.q.fy0 + (t / a.q.TW) * a.q.fsy;
                 raw = f2u(base[(((int64_t)(a.q.KH - 1 - fy) * a.q.KW + (a.q.KW - 1 - fx)) * a.q.IC + j) * a.q.OC + oc]);
             }
         }
@@ -607,7 +618,7 @@ void lutgemm_kernel(KArgs a)
     if (!active) return;
     if (seg_nsplit == 1) {
         if (r < a.R) {
-            float *o = a.out + (int64_t)bz * a.out_batch_stride + r * a.so_r;
+            float *o = a.out + (int64_t)bz * a.out_batch_stride + out_row_offset(a.ep.omap, r, a.so_r);
             if (a.ep.bias_j || a.ep.bias_r || a.ep.act) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
@@ -671,9 +682,19 @@ __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
         float s = part[0][o];
 #pragma unroll
         for (int w = 1; w < WAYS; ++w) s += part[w][o];
-        a.out[(int64_t)bz * a.out_batch_stride + (a.row_base + r) * a.so_r + j * a.so_j] =
+        a.out[(int64_t)bz * a.out_batch_stride + out_row_offset(a.ep.omap, a.row_base + r, a.so_r) + j * a.so_j] =
             apply_epilogue(a.ep, s, a.row_base + r, j);
     }
+}
+
+// Empty reduction: every output is the epilogue of zero (zeros without one).
+__global__ __launch_bounds__(WG_THREADS) void fill_empty_kernel(RArgs a)
+{
+    const int64_t idx = (int64_t)blockIdx.x * WG_THREADS + threadIdx.x;
+    if (idx >= a.R * a.J) return;
+    const int64_t r = idx / a.J, j = idx - r * a.J;
+    a.out[(int64_t)blockIdx.y * a.out_batch_stride + out_row_offset(a.ep.omap, a.row_base + r, a.so_r) + j * a.so_j] =
+        apply_epilogue(a.ep, 0.0f, a.row_base + r, j);
 }
 
 static void launch_reduce(const RArgs &ra, hipStream_t stream)
@@ -892,17 +913,18 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
         RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0,
-                 Epilogue{d.bias_j, d.bias_r, d.act}};
+                 Epilogue{d.bias_j, d.bias_r, d.act, d.omap}};
         if (d.batch > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
-        launch_reduce(ra, stream);
+        fill_empty_kernel<<<dim3((unsigned)((d.R * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch), WG_THREADS, 0,
+                            stream>>>(ra);
         AMSIM_HIP_CHECK(hipGetLastError());
         return AMSIM_OK;
     }
     if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
-    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, g_split_k.load() != 0);
+    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, g_split_k.load() != 0 && !d.no_split);
     // the size the query returns (valid for either split mode), not just this plan's
-    const size_t need = gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
+    const size_t need = d.no_split ? pl.total : gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
     if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need)
         return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
                                              std::to_string(need) + " bytes");
@@ -931,7 +953,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.Jp = pl.Jp; ka.nchunks = pl.nchunks;
     ka.out = d.out; ka.so_r = d.so_r; ka.so_j = d.so_j; ka.out_batch_stride = d.out_batch_stride;
     ka.batch = d.batch;
-    ka.ep = Epilogue{d.bias_j, d.bias_r, d.act};
+    ka.ep = Epilogue{d.bias_j, d.bias_r, d.act, d.omap};
 
     const int rows = 64 * pl.WR, wc = 4 / pl.WR;
     const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;

@@ -81,9 +81,18 @@ struct QDesc {
     int batches = 1;  // 1 = shared by every batch item
     // Q_DENSE: element (k, j) at base[k * sk + j * sj]
     int64_t sk = 0, sj = 0;
-    // Q_FLIP: k = (fy, fx, oc), j = ic of an HWIO filter [KH, KW, IC, OC]:
+    // Q_FLIP: k = (ty, tx, oc) over [TH, TW, OC], j = ic of an HWIO filter [KH, KW, IC, OC] read
+    //         flipped, every (fsy, fsx)-th tap from (fy0, fx0): fy = fy0 + ty * fsy, fx = fx0 + tx * fsx,
     //         base[((KH-1-fy) * KW + (KW-1-fx)) * IC * OC + ic * OC + oc]
     int KH = 0, KW = 0, IC = 0, OC = 0;
+    int TH = 0, TW = 0, fy0 = 0, fx0 = 0, fsy = 1, fsx = 1;
+};
+
+// Optional scatter of the output rows: row r = (b, y, x) over [B, GH, GW] is stored at pixel
+// (b, y * sy + oy, x * sx + ox) of a [B, H, W] image (so_r elements per pixel).
+struct OutMap {
+    int enabled = 0;
+    int GH = 0, GW = 0, sy = 1, sx = 1, oy = 0, ox = 0, H = 0, W = 0;
 };
 
 struct GemmDesc {
@@ -98,6 +107,8 @@ struct GemmDesc {
     // dimension carries the output channels), then the activation
     const float *bias_j = nullptr, *bias_r = nullptr;
     int act = AMSIM_ACT_NONE;
+    OutMap omap;
+    bool no_split = false;  // keep every reduction whole (needs no partial-sum workspace)
 };
 
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches);

@@ -136,7 +136,8 @@ def convam_input_grad(lut, input_sizes, filter, out_backprop, strides=(1, 1), pa
     hole_h = (oh - 1) * strides[0] + 1 if oh > 0 else 0
     hole_w = (ow - 1) * strides[1] + 1 if ow > 0 else 0
     lib = load_library()
-    nbytes = lib.amsim_convam_input_grad_workspace_bytes(n, h, wd, c, kh, kw, oc)
+    nbytes = lib.amsim_convam_input_grad_strided_workspace_bytes(n, h, wd, c, kh, kw, oc, strides[0], strides[1],
+                                                                 kh - 1 - pt, kw - 1 - pl)
     ws, wsp = _workspace(nbytes, dy.device)
     check(lib.amsim_convam_input_grad_f32(lut.handle, _ptr(dy), hole_w, hole_h, kh - 1 - pt, kw - 1 - pl, _ptr(w),
                                           kh, kw, oc, strides[0], strides[1], n, h, wd, c, _ptr(out), oh, ow,

@@ -139,6 +139,13 @@ int amsim_convam_bias_act_f32(amsim_lut_t lut, const float *input_data, float *o
  * stride-dilated gradient extent (convam.cc:1066-1067). */
 size_t amsim_convam_input_grad_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
                                                int filter_rows, int filter_cols, int out_depth);
+/* With strides above 1 the call runs one undilated sub-problem per residue class of the input
+ * pixels modulo the stride (the gradient's inserted zeros are never multiplied).  The query
+ * above does not know the strides; a workspace of the size below lets every sub-problem use its
+ * best split of the reduction (with less, sub-problems that would need more run unsplit). */
+size_t amsim_convam_input_grad_strided_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
+                                                       int filter_rows, int filter_cols, int out_depth,
+                                                       int stride_rows, int stride_cols, int pad_top, int pad_left);
 int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_grad_width, int hole_grad_height,
                                 int pad_top, int pad_left, const float *filter, int filter_rows,
                                 int filter_cols, int out_depth, int stride_rows, int stride_cols, int batch,
