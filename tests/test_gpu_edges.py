@@ -132,3 +132,63 @@ def test_runs_on_a_non_default_stream():
         out = functors.gemm(lut, Ad, Bd)
     s.synchronize()
     assert np.array_equal(host(out).view(np.uint32), cpu.gemm(lut32("MBM", 7), 7, A, B).view(np.uint32))
+
+
+@pytest.mark.parametrize("xs,ws,stride,padding", [((2, 9, 8, 16), (1, 1, 16, 24), 2, "SAME"),     # taps reach 1 pixel in 4
+                                                   ((2, 11, 7, 4), (2, 2, 4, 6), 3, "VALID"),      # filter smaller than stride
+                                                   ((1, 12, 12, 32), (3, 3, 32, 32), 2, "SAME"),
+                                                   ((3, 10, 13, 8), (5, 3, 8, 12), (2, 3), "SAME")])
+def test_strided_grad_input_residue_classes(xs, ws, stride, padding):
+    """Grad-input with strides above 1 runs one sub-problem per residue class of the input pixels:
+    same bits as the oracle's dilated-gradient loop nest, zeros where no tap reaches."""
+    import approxtrain_amd
+    from approxtrain_amd import ApproxMulLut, functors
+    approxtrain_amd.load_library().amsim_set_split_k(0)
+    try:
+        lut = ApproxMulLut.cached(lut_path("MBM", 7))
+        L = lut32("MBM", 7)
+        st = (stride, stride) if isinstance(stride, int) else stride
+        rng = np.random.default_rng(sum(xs))
+        w = rng.standard_normal(ws).astype(np.float32)
+        oh, _ = cpu.conv_geometry(xs[1], ws[0], st[0], padding)
+        ow, _ = cpu.conv_geometry(xs[2], ws[1], st[1], padding)
+        dy = rng.standard_normal((xs[0], oh, ow, ws[3])).astype(np.float32)
+        got = host(functors.convam_input_grad(lut, xs, dev(w), dev(dy), st, padding))
+        want = cpu.conv2d_grad_input(L, 7, xs, w, dy, st, padding)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    finally:
+        approxtrain_amd.load_library().amsim_set_split_k(1)
+
+
+def test_strided_grad_input_with_the_stride_agnostic_workspace():
+    """A caller that sizes the workspace with the reference-shaped query (no strides) still gets the
+    right answer: sub-problems that would want more room run with their reductions whole."""
+    import approxtrain_amd
+    from approxtrain_amd import ApproxMulLut
+    lib = approxtrain_amd.load_library()
+    lib.amsim_set_split_k(1)  # splitting allowed: the two workspace sizes then lead to different plans
+    lut = ApproxMulLut.cached(lut_path("MBM", 7))
+    n, h, w_, c, kh, kw, oc, s = 4, 28, 28, 64, 3, 3, 64, 2
+    oh = ow = 14
+    rng = np.random.default_rng(12)
+    filt = rng.standard_normal((kh, kw, c, oc)).astype(np.float32)
+    dy = rng.standard_normal((n, oh, ow, oc)).astype(np.float32)
+    small = lib.amsim_convam_input_grad_workspace_bytes(n, h, w_, c, kh, kw, oc)
+    big = lib.amsim_convam_input_grad_strided_workspace_bytes(n, h, w_, c, kh, kw, oc, s, s, kh - 1 - 0, kw - 1 - 0)
+    assert big >= small
+    outs = []
+    for nbytes in (small, big):
+        ws = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda")
+        base = ws.data_ptr() + (-ws.data_ptr()) % 256
+        out = torch.full((n, h, w_, c), 7.0, device="cuda")
+        fd, gd = dev(filt), dev(dy)
+        # SAME, stride 2, 28 -> 14: total padding 1, forward pad_top = 0 -> back pad = kh - 1
+        rc = lib.amsim_convam_input_grad_f32(lut.handle, C.c_void_p(gd.data_ptr()), (ow - 1) * s + 1, (oh - 1) * s + 1,
+                                             kh - 1, kw - 1, C.c_void_p(fd.data_ptr()), kh, kw, oc, s, s, n, h, w_, c,
+                                             C.c_void_p(out.data_ptr()), oh, ow, C.c_void_p(base), nbytes, None)
+        assert rc == 0, lib.amsim_last_error()
+        outs.append(host(out))
+    want = cpu.conv2d_grad_input(lut32("MBM", 7), 7, (n, h, w_, c), filt, dy, (s, s), "SAME")
+    sum_abs = np.abs(want).max() * 50 + 1.0
+    for got in outs:
+        assert np.all(np.abs(got - want) <= 1e-5 * sum_abs)
