@@ -36,7 +36,6 @@ struct Lut {
     uint8_t *img_ab = nullptr;
     uint8_t *img_ba = nullptr;
     uint32_t *lut32 = nullptr;
-    uint32_t *lut32_t = nullptr;  // transposed 32-bit table
     // m > 7 only: carry << 15 | mantissa << (15 - m), and its transpose
     uint16_t *img16_ab = nullptr;
     uint16_t *img16_ba = nullptr;

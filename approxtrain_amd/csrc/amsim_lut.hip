@@ -23,24 +23,32 @@ int fail(int status, const std::string &msg)
 const std::string &last_error() { return g_last_error; }
 
 // entries: one (carry, mantissa) pair per (ma, mb), mantissa in m bits
+void lut_free(Lut &l);
+
 static int build_images(int m, const std::vector<uint8_t> &carry, const std::vector<uint32_t> &mant, Lut *out)
 {
     const size_t n = (size_t)1 << m, total = n * n;
-    std::vector<uint32_t> l32(total), l32t(total);
-    for (size_t i = 0; i < n; ++i)
-        for (size_t j = 0; j < n; ++j) {
-            const uint32_t v = ((uint32_t)carry[i * n + j] << 23) | (mant[i * n + j] << (23 - m));
-            l32[i * n + j] = v;
-            l32t[j * n + i] = v;
-        }
     Lut l;
     l.m = m;
     l.entries = total;
     AMSIM_HIP_CHECK(hipGetDevice(&l.device));
-    AMSIM_HIP_CHECK(hipMalloc(&l.lut32, total * 4));
-    AMSIM_HIP_CHECK(hipMemcpy(l.lut32, l32.data(), total * 4, hipMemcpyHostToDevice));
-    AMSIM_HIP_CHECK(hipMalloc(&l.lut32_t, total * 4));
-    AMSIM_HIP_CHECK(hipMemcpy(l.lut32_t, l32t.data(), total * 4, hipMemcpyHostToDevice));
+    // device copy of a host vector; on failure everything uploaded so far is released
+    auto upload = [&](auto **dst, const auto &host) -> int {
+        const size_t bytes = host.size() * sizeof(host[0]);
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(dst), bytes);
+        if (e == hipSuccess) e = hipMemcpy(*dst, host.data(), bytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            lut_free(l);
+            return fail(AMSIM_ERR_HIP, std::string("LUT upload: ") + hipGetErrorString(e));
+        }
+        return AMSIM_OK;
+    };
+    int rc;
+    {
+        std::vector<uint32_t> l32(total);
+        for (size_t i = 0; i < total; ++i) l32[i] = ((uint32_t)carry[i] << 23) | (mant[i] << (23 - m));
+        if ((rc = upload(&l.lut32, l32)) != AMSIM_OK) return rc;
+    }
     if (m <= 7) {
         // + one all-zero row of n entries after the table (selected by zero operands)
         const size_t padded = (total + n + 15) / 16 * 16;
@@ -51,12 +59,9 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
                 ab[i * n + j] = b;
                 ba[j * n + i] = b;
             }
-        AMSIM_HIP_CHECK(hipMalloc(&l.img_ab, padded));
-        AMSIM_HIP_CHECK(hipMemcpy(l.img_ab, ab.data(), padded, hipMemcpyHostToDevice));
-        AMSIM_HIP_CHECK(hipMalloc(&l.img_ba, padded));
-        AMSIM_HIP_CHECK(hipMemcpy(l.img_ba, ba.data(), padded, hipMemcpyHostToDevice));
-    }
-    if (m > 7) {
+        if ((rc = upload(&l.img_ab, ab)) != AMSIM_OK) return rc;
+        if ((rc = upload(&l.img_ba, ba)) != AMSIM_OK) return rc;
+    } else {
         std::vector<uint16_t> ab(total + n, 0), ba(total + n, 0);  // + the all-zero row
         for (size_t i = 0; i < n; ++i)
             for (size_t j = 0; j < n; ++j) {
@@ -64,10 +69,8 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
                 ab[i * n + j] = b;
                 ba[j * n + i] = b;
             }
-        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ab, (total + n) * 2));
-        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ab, ab.data(), (total + n) * 2, hipMemcpyHostToDevice));
-        AMSIM_HIP_CHECK(hipMalloc(&l.img16_ba, (total + n) * 2));
-        AMSIM_HIP_CHECK(hipMemcpy(l.img16_ba, ba.data(), (total + n) * 2, hipMemcpyHostToDevice));
+        if ((rc = upload(&l.img16_ab, ab)) != AMSIM_OK) return rc;
+        if ((rc = upload(&l.img16_ba, ba)) != AMSIM_OK) return rc;
     }
     *out = l;
     return AMSIM_OK;
@@ -109,7 +112,6 @@ void lut_free(Lut &l)
     if (l.img_ab) (void)hipFree(l.img_ab);
     if (l.img_ba) (void)hipFree(l.img_ba);
     if (l.lut32) (void)hipFree(l.lut32);
-    if (l.lut32_t) (void)hipFree(l.lut32_t);
     if (l.img16_ab) (void)hipFree(l.img16_ab);
     if (l.img16_ba) (void)hipFree(l.img16_ba);
     l = Lut{};
