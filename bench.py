@@ -60,6 +60,25 @@ def measure_peaks(lib, cus):
     return out
 
 
+def profiled_traffic():
+    """HBM bytes per launch of the forward kernel from the committed rocprofv3 counter summary
+    (FETCH_SIZE / WRITE_SIZE runs scaled by the calibration copy; see the file for the commands).
+    The counters cannot be read from inside this process, so the figure is the last profiled one."""
+    path = os.path.join(ROOT, "profiles", "lutgemm_conv3x3_resnet50_mbm7.txt")
+    try:
+        lines = open(path).read().split("\n")
+        start = next(i for i, l in enumerate(lines) if l.startswith("== HBM traffic counters"))
+        for l in lines[start:]:
+            if l.startswith("lutgemm_kernel<16, 1, 1,"):
+                read_mib, written_mib = (float(v) for v in l.split()[-2:])
+                return {"bytes": int((read_mib + written_mib) * 2 ** 20), "read_bytes": int(read_mib * 2 ** 20),
+                        "written_bytes": int(written_mib * 2 ** 20),
+                        "source": "profiles/lutgemm_conv3x3_resnet50_mbm7.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"}
+    except (OSError, StopIteration, ValueError):
+        pass
+    return None
+
+
 def cpu_baseline(x, w, dy):
     """The CPU oracle (a port of the reference's loop nests with the LUT
     product) on a bounded sample: the first image of the batch, all three
@@ -180,7 +199,7 @@ def main():
             "measured_peaks": {k: round(v / 1e12, 3) for k, v in peaks.items()}, "measured_peaks_unit": "T/s",
             "hbm": {"algorithmic_bytes": alg_bytes, "achieved_GBps": round(alg_bytes / (pass_ms["fwd"] * 1e-3) / 1e9, 1),
                     "peak_GBps": 8000.0},
-            "traffic": None,
+            "traffic": profiled_traffic(),
         },
     }
     if not args.no_cpu_baseline:
