@@ -99,6 +99,7 @@ struct KArgs {
     float *out;
     int64_t so_r, so_j, out_batch_stride;
     int batch;
+    int vec_store;           // outputs of a row are contiguous (so_j == 1) and every row starts 16-byte aligned
     Epilogue ep;
     // A launch covers up to two row segments, workgroups of seg[0] first in dispatch order:
     // seg[0] the split-reduction tail (if any), seg[1] the main part.
@@ -621,8 +622,13 @@ void lutgemm_kernel(KArgs a)
             float *o = a.out + (int64_t)bz * a.out_batch_stride + out_row_offset(a.ep.omap, r, a.so_r);
             if (a.ep.bias_j || a.ep.bias_r || a.ep.act) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    if (j0 + j < a.J) o[(int64_t)(j0 + j) * a.so_j] = apply_epilogue(a.ep, acc[j], r, j0 + j);
+                for (int j = 0; j < TN; ++j) acc[j] = apply_epilogue(a.ep, acc[j], r, min((int64_t)(j0 + j), a.J - 1));
+            }
+            if (TN % 4 == 0 && a.vec_store && j0 + TN <= a.J) {
+                // a lane's TN outputs are contiguous and 16-byte aligned: whole float4 stores
+                float4 *o4 = reinterpret_cast<float4 *>(o + j0);
+#pragma unroll
+                for (int j = 0; j < TN / 4; ++j) o4[j] = make_float4(acc[4 * j], acc[4 * j + 1], acc[4 * j + 2], acc[4 * j + 3]);
             } else {
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
@@ -954,6 +960,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.out = d.out; ka.so_r = d.so_r; ka.so_j = d.so_j; ka.out_batch_stride = d.out_batch_stride;
     ka.batch = d.batch;
     ka.ep = Epilogue{d.bias_j, d.bias_r, d.act, d.omap};
+    ka.vec_store = (d.so_j == 1 && d.so_r % 4 == 0 && d.out_batch_stride % 4 == 0 && aligned16(d.out)) ? 1 : 0;
 
     const int rows = 64 * pl.WR, wc = 4 / pl.WR;
     const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;
