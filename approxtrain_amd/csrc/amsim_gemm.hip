@@ -797,29 +797,30 @@ static Shape shape_work(int64_t rowtiles, int64_t G, int n, int64_t slots, bool 
     return best;
 }
 
-static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k);
+static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64);
 
 // Plans are pure functions of their arguments; the last few are remembered per thread so that
 // the workspace query and the call that follows it do not repeat the search.
-static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k)
+// waves64: waves per SIMD the 64-row kernel variant that will run is compiled for
+static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64)
 {
     struct Key { int64_t R, J, K; int batch, qb, split; };
     struct Slot { Key k; Plan p; bool used = false; };
     static thread_local Slot memo[8];
     static thread_local unsigned next = 0;
-    const Key key{R, J, K, batch, q_batches, split_k ? 1 : 0};
+    const Key key{R, J, K, batch, q_batches, (split_k ? 1 : 0) | (waves64 << 1)};
     for (const Slot &sl : memo)
         if (sl.used && sl.k.R == R && sl.k.J == J && sl.k.K == K && sl.k.batch == batch && sl.k.qb == q_batches &&
             sl.k.split == key.split)
             return sl.p;
     Slot &sl = memo[next++ % 8];
     sl.k = key;
-    sl.p = compute_plan(R, J, K, batch, q_batches, split_k);
+    sl.p = compute_plan(R, J, K, batch, q_batches, split_k, waves64);
     sl.used = true;
     return sl.p;
 }
 
-static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k)
+static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64)
 {
     Plan pl{};
     // Narrow outputs (one column group) stack four row tiles per workgroup and shrink the
@@ -834,7 +835,7 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
     pl.Rp = (R + rows - 1) / rows * rows;
     const int64_t rowtiles = pl.Rp / rows;
     const int64_t G = ((jchunks + wc - 1) / wc) * batch;
-    const int64_t slots = pl.WR == 1 ? WG_SLOTS : DEVICE_CUS * 2;  // resident workgroups (the 256-row kernels run 2 per CU)
+    const int64_t slots = DEVICE_CUS * (pl.WR == 1 ? waves64 : 2);  // resident workgroups (the 256-row kernels run 2 per CU)
 
     Shape sh;
     sh.cps = pl.nchunks;
@@ -870,25 +871,44 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 {
     if (R <= 0 || J <= 0 || K <= 0 || batch <= 0) return 0;
-    // valid whichever way amsim_set_split_k stands when the call is made
-    return std::max(make_plan(R, J, K, batch, q_batches, true).total, make_plan(R, J, K, batch, q_batches, false).total);
+    // valid whichever way amsim_set_split_k stands when the call is made and whichever kernel
+    // variant (6 or 5 waves per SIMD) the operand layout selects
+    size_t need = make_plan(R, J, K, batch, q_batches, false, WAVES_PER_SIMD).total;
+    for (int w = WAVES_PER_SIMD - 1; w <= WAVES_PER_SIMD; ++w)
+        need = std::max(need, make_plan(R, J, K, batch, q_batches, true, w).total);
+    return need;
 }
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// staging mode of the lane operand for a problem (which kernel variant runs)
+static int stage_of(const PDesc &p, int64_t K)
+{
+    if (p.kind == P_DENSE) {
+        const bool k_contig = p.sk == 1 && p.sr != 1;
+        const bool vec = k_contig && (p.sr % 4 == 0) && (K % 4 == 0) && (p.batch_stride % 4 == 0) && aligned16(p.base);
+        return vec ? STAGE_K4 : k_contig ? STAGE_K : STAGE_R;
+    }
+    if (p.kind == P_PATCH) return ((p.C % 4 == 0) && aligned16(p.base)) ? STAGE_K4 : STAGE_K;
+    return STAGE_R;
+}
+// waves per SIMD the 64-row variant of that problem is compiled for (its __launch_bounds__)
+static int waves64_of(const PDesc &p, int64_t K)
+{
+    return (p.kind == P_DENSE && stage_of(p, K) != STAGE_K4) ? WAVES_PER_SIMD - 1 : WAVES_PER_SIMD;
+}
 
 template <int TN, int WR, bool LUTG>
 static void launch_variant(const KArgs &ka, dim3 grid, hipStream_t stream)
 {
     const PDesc &p = ka.p;
+    const int stage = stage_of(p, ka.K);
     if (p.kind == P_DENSE) {
-        const bool k_contig = p.sk == 1 && p.sr != 1;
-        const bool vec = k_contig && (p.sr % 4 == 0) && (ka.K % 4 == 0) && (p.batch_stride % 4 == 0) && aligned16(p.base);
-        if (vec) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K4, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
-        else if (k_contig) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
+        if (stage == STAGE_K4) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K4, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
+        else if (stage == STAGE_K) lutgemm_kernel<TN, WR, P_DENSE, STAGE_K, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
         else lutgemm_kernel<TN, WR, P_DENSE, STAGE_R, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
     } else if (p.kind == P_PATCH) {
-        const bool vec = (p.C % 4 == 0) && aligned16(p.base);
-        if (vec) lutgemm_kernel<TN, WR, P_PATCH, STAGE_K4, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
+        if (stage == STAGE_K4) lutgemm_kernel<TN, WR, P_PATCH, STAGE_K4, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
         else lutgemm_kernel<TN, WR, P_PATCH, STAGE_K, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
     } else {
         lutgemm_kernel<TN, WR, P_GF, STAGE_R, LUTG><<<grid, WG_THREADS, 0, stream>>>(ka);
@@ -928,7 +948,8 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     }
     if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
-    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, g_split_k.load() != 0 && !d.no_split);
+    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, g_split_k.load() != 0 && !d.no_split,
+                              waves64_of(d.p, d.K));
     // the size the query returns (valid for either split mode), not just this plan's
     const size_t need = d.no_split ? pl.total : gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
     if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need)
