@@ -37,6 +37,7 @@ SIGNATURES = {
     "amsim_lut_generate_builtin": (_i, [C.c_char_p, _i, _i, _p, _sz]),
     "amsim_mul_f32": (_i, [_p, _f, _f, _f, _sz, _p]),
     "amsim_gemm_workspace_bytes": (_sz, [_i, _i, _i64, _i64, _i64, _i64]),
+    "amsim_gemm_plan_info": (_i, [_i, _i, _i64, _i64, _i64, _i64, C.POINTER(_i64)]),
     "amsim_gemm_f32": (_i, [_p, _i, _i, _i, _i64, _i64, _i64, _f, _i64, _f, _i64, _f, _i64,
                             _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "amsim_convam_workspace_bytes": (_sz, [_i] * 7),

@@ -23,9 +23,14 @@ inline int64_t padded_work(int64_t R, int64_t J)
 }
 
 // true: rows of C over the lanes (lane operand = op(A)); false: columns of C
-// over the lanes (lane operand = op(B)).  Picks the orientation that wastes
-// fewer lanes / accumulators on padding.
-inline bool lanes_along_m(int64_t M, int64_t N) { return padded_work(M, N) <= padded_work(N, M); }
+// over the lanes (lane operand = op(B)).  Picks the cheaper orientation: the MACs spent
+// including lanes / accumulators wasted on padding (~13 TMAC/s), plus the pre-decode of the
+// uniform operand, which moves about 12 bytes per element (~4 TB/s).
+inline double orientation_cost(int64_t R, int64_t J, int64_t K)
+{
+    return (double)padded_work(R, J) * (double)K / 13.0e12 + 12.0 * (double)K * (double)J / 4.0e12;
+}
+inline bool lanes_along_m(int64_t M, int64_t N, int64_t K) { return orientation_cost(M, N, K) <= orientation_cost(N, M, K); }
 
 struct GemmCall {
     int transA, transB, swap;
@@ -45,7 +50,7 @@ GemmDesc describe(const GemmCall &g)
     d.batch = (int)g.batch;
     d.out = g.C;
     d.out_batch_stride = g.strideC;
-    if (lanes_along_m(g.M, g.N)) {
+    if (lanes_along_m(g.M, g.N, g.K)) {
         d.R = g.M; d.J = g.N;
         d.p.kind = P_DENSE; d.p.base = g.A; d.p.batch_stride = g.strideA;
         d.p.sr = g.transA ? 1 : g.lda; d.p.sk = g.transA ? g.lda : 1;
@@ -116,6 +121,16 @@ size_t amsim_gemm_workspace_bytes(int transA, int transB, int64_t M, int64_t N, 
     // sized for per-item operands (no broadcast), the larger case
     GemmCall g{transA, transB, 0, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, batch, 1, 1, 1};
     return gemm_ws(g);
+}
+
+int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t info[8])
+{
+    if (!info || M <= 0 || N <= 0 || K <= 0 || batch <= 0) return fail(AMSIM_ERR_INVALID, "bad plan query");
+    GemmCall g{transA, transB, 0, M, N, K, nullptr, transA ? M : K, nullptr, transB ? K : N, nullptr, N, batch, 1, 1, 1};
+    const GemmDesc d = describe(g);
+    // contiguous, aligned operands assumed (the float4-staged kernel variants)
+    gemm_plan_info(d.R, d.J, d.K, d.batch, d.q.batches, true, d.p.sk == 1 && d.p.sr != 1 ? 6 : 5, info);
+    return AMSIM_OK;
 }
 
 int amsim_gemm_f32(amsim_lut_t lut, int transA, int transB, int swap_operands, int64_t M, int64_t N, int64_t K,

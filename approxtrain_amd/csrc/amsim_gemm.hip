@@ -879,6 +879,16 @@ size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
     return need;
 }
 
+// what the planner decides for a problem: {TN, WR, nsplit, chunks per split, rows of the main
+// part, tail nsplit, tail chunks per split, chunks} (for tests and tuning)
+void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int64_t info[8])
+{
+    const Plan pl = make_plan(R, J, K, batch, q_batches, split_k, waves64);
+    info[0] = pl.TN; info[1] = pl.WR; info[2] = pl.nsplit; info[3] = pl.chunks_per_split;
+    info[4] = pl.rows_main; info[5] = pl.rows_main < R ? pl.tail_nsplit : 0;
+    info[6] = pl.rows_main < R ? pl.tail_chunks_per_split : 0; info[7] = pl.nchunks;
+}
+
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // staging mode of the lane operand for a problem (which kernel variant runs)

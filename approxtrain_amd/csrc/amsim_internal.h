@@ -111,6 +111,7 @@ struct GemmDesc {
 };
 
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
+void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int64_t info[8]);
 int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream);
 
 int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream);

@@ -199,6 +199,11 @@ int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, i
  * output (bit-identical to a sequential CPU loop); 1 (default) lets problems
  * with few outputs split the reduction across workgroups. */
 int amsim_set_split_k(int mode);
+/* How a GEMM of this shape would be run when reductions may be split (contiguous, aligned
+ * operands assumed): info = {outputs per lane, row tiles per workgroup, splits of the main part's
+ * reduction, chunks (of 32) per split, rows in the main part, splits of the tail rows' reduction
+ * (0 = no tail), chunks per tail split, chunks in all}.  For tests and tuning. */
+int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t info[8]);
 /* Micro-kernels that measure, on the current device, the VALU issue rate
  * (kind 0 / 10: independent FP32 FMAs; 11..13: v_add_u32, v_lshl_add_u32,
  * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's 3-op per-MAC mix) and

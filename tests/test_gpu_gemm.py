@@ -236,3 +236,41 @@ def test_generated_table_files_load_and_multiply(amd, tmp_path):
         got = host(amd.gemm(lut, dev(A), dev(B)))
         want = cpu.gemm(cpu.lutgen32(kind, m), m, A, B)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def _plan(M, N, K, batch=1, ta=0, tb=0):
+    import ctypes as C
+    import approxtrain_amd
+    info = (C.c_int64 * 8)()
+    assert approxtrain_amd.load_library().amsim_gemm_plan_info(ta, tb, M, N, K, batch, info) == 0
+    return dict(zip(("TN", "WR", "nsplit", "cps", "rows_main", "tail_nsplit", "tail_cps", "chunks"), info))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,expect", [
+    (100352, 64, 576, "tail"),          # one round and a bit: unsplit main part + split tail
+    (25088, 128, 1152, "split+tail"),   # half a round: main part split in two, tail split further
+    (6272, 256, 2304, "split+tail"),
+    (512, 512, 8192, "split"),          # few outputs, long reduction
+    (51200, 64, 128, "whole"),          # short reduction: nothing to gain from splitting
+    (40, 6, 50000, "split"),            # one row tile
+])
+def test_planner_paths_match_the_oracle(amd, M, N, K, expect):
+    """The work-shaping decisions (reduction split, tail rows split further, both with partial sums)
+    at shapes that take each path: result within 1e-5 * sum|products| of the sequential oracle."""
+    from approxtrain_amd import ApproxMulLut
+    p = _plan(M, N, K)
+    split, tail = p["nsplit"] > 1, p["tail_nsplit"] > 0
+    assert {"tail": (not split) and tail, "split+tail": split and tail, "split": split and not tail,
+            "whole": (not split) and (not tail)}[expect], p
+    _set_split(1)
+    rng = np.random.default_rng(M + N + K)
+    # a sample of the rows keeps the oracle fast: the GPU computes everything, rows are independent
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    lut = ApproxMulLut.cached(lut_path("MBM", 7))
+    got = host(amd.gemm(lut, dev(A), dev(B)))
+    rows = np.unique(np.concatenate([np.arange(min(M, 70)), rng.integers(0, M, 60), np.arange(max(M - 130, 0), M)]))
+    L = lut32("MBM", 7)
+    want = cpu.gemm(L, 7, A[rows].copy(), B)
+    assert_close_sum_abs(got[rows], want, cpu.gemm_abs(L, 7, A[rows].copy(), B), 1e-5)
