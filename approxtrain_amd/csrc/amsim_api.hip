@@ -316,11 +316,25 @@ int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_gra
     return AMSIM_OK;
 }
 
+namespace {
+// A 1x1 filter at stride 1 without padding makes the filter gradient the plain product
+// input^T [C x K] . grad [K x OC]: either operand may then be the pre-decoded one.
+GemmCall pointwise_filter_grad(int64_t pixels, int in_depth, int out_depth, const float *input, const float *grad,
+                               float *output)
+{
+    return GemmCall{1, 0, 0, in_depth, out_depth, pixels, input, in_depth, grad, out_depth, output, out_depth, 1, 0, 0, 0};
+}
+}  // namespace
+
 size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth,
                                                 int filter_rows, int filter_cols, int in_depth)
 {
-    return gemm_workspace_bytes((int64_t)filter_rows * filter_cols * in_depth, out_depth,
-                                (int64_t)batch * out_rows * out_cols, 1, 1);
+    size_t need = gemm_workspace_bytes((int64_t)filter_rows * filter_cols * in_depth, out_depth,
+                                       (int64_t)batch * out_rows * out_cols, 1, 1);
+    if (filter_rows == 1 && filter_cols == 1)
+        need = std::max(need, gemm_ws(pointwise_filter_grad((int64_t)batch * out_rows * out_cols, in_depth, out_depth,
+                                                            nullptr, nullptr, nullptr)));
+    return need;
 }
 
 int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const float *grad, int input_rows,
@@ -340,6 +354,10 @@ int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const floa
     if (K > 0 && (!input || !grad)) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
     if (!fits_int32((int64_t)batch * input_rows * input_cols * in_depth))
         return fail(AMSIM_ERR_UNSUPPORTED, "input tensor has 2^31 or more elements");
+    if (filter_rows == 1 && filter_cols == 1 && stride_rows == 1 && stride_cols == 1 && filter_top_offset == 0 &&
+        filter_left_offset == 0 && out_rows == input_rows && out_cols == input_cols)
+        return gemm_call(lut, pointwise_filter_grad(K, in_depth, out_depth, input, grad, output), workspace,
+                         workspace_bytes, stream);  // P(input, grad), reduction over (b, oy, ox) as below
     // rows (fy, fx, c) of the filter x reduction over (b, oy, ox)
     // [cuda_kernel.cu:327-353, 417-425]; the gradient is the [K][OC] matrix
     GemmDesc d;
