@@ -38,6 +38,15 @@ struct SafeRange {
     __device__ __forceinline__ bool unsafe() const { return tmax >= (191u << 24) || tmin < (64u << 24) - 1u; }
 };
 
+// 64-bit add of a vector register pair and a scalar register pair in one instruction (the
+// compiler's own choice for this sum is a multiply-add form that issues several times slower).
+__device__ __forceinline__ uint64_t add_u64_vs(uint64_t v, uint64_t s_uniform)
+{
+    uint64_t d;
+    asm("v_lshl_add_u64 %0, %1, 0, %2" : "=v"(d) : "v"(v), "s"(s_uniform));
+    return d;
+}
+
 // Full-domain product.  `entry16` is the LUT byte (carry << 7 | mantissa
 // left-aligned in 7 bits) shifted left by 16, i.e. carry << 23 | mantissa.
 // Restates the exponent / special-case logic of the C functional models:
