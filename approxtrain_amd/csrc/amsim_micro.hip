@@ -13,8 +13,8 @@ constexpr int MICRO_UNROLL = 16;
 
 // VMODE 0: v_fma_f32   1: v_add_u32   2: v_lshl_add_u32   3: v_mul_f32
 //       4: a 4-op mix (add, mul, lshl_add, fma)
-//       5: the GEMM's per-MAC mix: v_or_b32 (SGPR | VGPR), v_lshl_add_u32 (VGPR << 16 + SGPR),
-//          v_fma_f32 -- 3 ops per slot
+//       5: the GEMM's mix per pair of MACs: one v_lshl_add_u64 (VGPR pair + SGPR pair, two LUT
+//          addresses), two v_lshl_add_u32 (VGPR << 16 + SGPR), two v_fma_f32 -- 5 ops per two slots
 template <int VMODE>
 __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, float *sink, long long *clk)
 {
@@ -22,6 +22,8 @@ __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, fl
 #pragma unroll
     for (int j = 0; j < MICRO_UNROLL; ++j) a[j] = (float)(threadIdx.x + j) * 1e-3f;
     float c1 = 0.999f + 1e-6f * threadIdx.x, c2 = 1e-3f;
+    const uint64_t pair = ((uint64_t)threadIdx.x << 32) | threadIdx.x;
+    const uint64_t spair = ((uint64_t)(uint32_t)iters << 32) | (uint32_t)iters;
     const long long t0 = clock64();
     for (int i = 0; i < iters; ++i) {
 #pragma unroll
@@ -31,10 +33,14 @@ __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, fl
             else if (VMODE == 2) asm volatile("v_lshl_add_u32 %0, %0, 16, %1" : "+v"(a[j]) : "v"(c1));
             else if (VMODE == 3) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(a[j]) : "v"(c1));
             else if (VMODE == 5) {
-                float t;
-                asm volatile("v_or_b32 %0, %1, %2" : "=v"(t) : "s"(iters), "v"(c1));
-                asm volatile("v_lshl_add_u32 %0, %1, 16, %2" : "=v"(t) : "v"(t), "s"(iters));
-                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j]) : "v"(c2), "v"(t));
+                if (j & 1) continue;  // slots are handled in pairs
+                uint64_t t2;
+                uint32_t t0, t1;
+                asm volatile("v_lshl_add_u64 %0, %1, 0, %2" : "=v"(t2) : "v"(pair), "s"(spair));
+                asm volatile("v_lshl_add_u32 %0, %1, 16, %2" : "=v"(t0) : "v"((uint32_t)t2), "s"(iters));
+                asm volatile("v_lshl_add_u32 %0, %1, 16, %2" : "=v"(t1) : "v"((uint32_t)(t2 >> 32)), "s"(iters));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j]) : "v"(c2), "v"(t0));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j + 1]) : "v"(c2), "v"(t1));
             } else {
                 float t, f;
                 asm volatile("v_add_u32 %0, %1, %2" : "=v"(t) : "v"(a[j]), "v"(c1));
@@ -162,7 +168,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
     AMSIM_HIP_CHECK(hipEventDestroy(e1));
     AMSIM_HIP_CHECK(hipGetLastError());
     *ms_per_launch = (double)ms / reps;
-    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4 : kind == 15 ? 3 : 1);
+    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4.0 : kind == 15 ? 2.5 : 1.0);
     return AMSIM_OK;
 }
 

@@ -26,7 +26,7 @@ METRIC = "approx GMAC/s + % VALU/LDS roofline, AMConv2D fwd+bwd ResNet-50 3x3, M
 LUT_FILE = os.path.join(ROOT, "tests", "golden", "lut", "MBM_7.bin")
 XS, WS = (32, 56, 56, 64), (3, 3, 64, 64)
 MACS_PER_PASS = 32 * 56 * 56 * 64 * 3 * 3 * 64  # 3 699 376 128
-VALU_OPS_PER_MAC = 3      # v_or (LUT address), v_lshl_add (byte -> product factor), v_fma in the kernel's inner loop
+VALU_OPS_PER_MAC = 2.5    # per two MACs: one v_lshl_add_u64 (two LUT addresses), two v_lshl_add_u32 (byte -> product factor), two v_fma
 NOMINAL_OPS_PER_MAC = 5   # the figure the roofline definition quotes as nominal
 
 

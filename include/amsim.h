@@ -206,7 +206,7 @@ int amsim_set_split_k(int mode);
 int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t info[8]);
 /* Micro-kernels that measure, on the current device, the VALU issue rate
  * (kind 0 / 10: independent FP32 FMAs; 11..13: v_add_u32, v_lshl_add_u32,
- * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's 3-op per-MAC mix) and
+ * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's mix, 5 instructions per two MACs) and
  * the LDS gather rate (kinds 1..6: u8 / u16 / b32 reads, lanes inside one
  * 128-element row or scattered).  Launches
  * `reps` times on `stream`, timed with HIP events; `sink` is any device buffer
