@@ -33,6 +33,21 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert sorted(_lib.SIGNATURES) == names
 
 
+def test_tensorflow_bridge_uses_only_declared_entry_points():
+    """The TensorFlow bridge cannot be compiled here (no TensorFlow); at least every C-ABI
+    call in it must name an entry point the header declares, and every GPU functor of the
+    reference must be defined and instantiated in it."""
+    text = open(os.path.join(ROOT, "approxtrain_amd", "tf_bridge", "amsim_tf_bridge.cc")).read()
+    code = re.sub(r"//.*", "", text)
+    used = set(re.findall(r"\b(amsim_[a-z0-9_]+)\s*\(", code))
+    assert used and used <= set(declared_symbols()), used - set(declared_symbols())
+    for functor in ("ConvamFunctor", "ConvamInputGradFunctor", "ConvamFilterGradFunctor", "DenseamFunctor",
+                    "DenseamWeightGradFunctor", "DenseamInputGradFunctor", "LaunchMatMul"):
+        assert re.search(r"void %s<GPUDevice, T>::operator\(\)" % functor, code), functor
+        for t in ("float", "int32"):
+            assert "template struct %s<GPUDevice, %s>;" % (functor, t) in code, (functor, t)
+
+
 def test_status_strings():
     lib = approxtrain_amd.load_library()
     assert lib.amsim_status_string(0) == b"ok"
