@@ -55,6 +55,10 @@ SIGNATURES = {
     "amsim_denseam_input_grad_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),
     "amsim_matmulam_workspace_bytes": (_sz, [_i] * 6),
     "amsim_matmulam_f32": (_i, [_p, _f, _f] + [_i] * 6 + [_f, _p, _sz, _p]),
+    "amsim_attention_workspace_bytes": (_sz, [_i] * 5),
+    "amsim_attention_f32": (_i, [_p, _f, _f, _f, _f, _i, _i64, _i64] + [_i] * 5 + [C.c_float, _f, _f, _p, _sz, _p]),
+    "amsim_attention_grad_workspace_bytes": (_sz, [_i] * 5),
+    "amsim_attention_grad_f32": (_i, [_p, _f, _f, _f, _f, _f] + [_i] * 5 + [C.c_float, _f, _f, _f, _p, _sz, _p]),
     "amsim_conv_geometry": (_i, [_i, _i, _i, _i, C.POINTER(_i), C.POINTER(_i)]),
     "amsim_set_split_k": (_i, [_i]),
     "amsim_calibration_copy": (_i, [_f, _f, _sz, _p]),

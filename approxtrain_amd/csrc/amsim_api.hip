@@ -455,6 +455,113 @@ int amsim_matmulam_f32(amsim_lut_t lut, const float *a, const float *b, int batc
     return gemm_call(lut, g, workspace, workspace_bytes, stream);
 }
 
+// ---- dot-product attention --------------------------------------------------------------
+// multihead_attention.py:18-30 on contiguous [batch][seq][depth] operands: two strided-batch
+// products around the row softmax.  Gradient wiring follows math_ops.py:141-157: the op never
+// sees the transpose flags, so every gradient is (grad, b_op^T) and (a_op^T, grad).
+
+namespace {
+
+struct AttnShape {
+    int batch, seq_q, seq_k, d_k, d_v;
+    int64_t nq() const { return (int64_t)seq_q * d_k; }
+    int64_t nk() const { return (int64_t)seq_k * d_k; }
+    int64_t nv() const { return (int64_t)seq_k * d_v; }
+    int64_t nw() const { return (int64_t)seq_q * seq_k; }
+    int64_t no() const { return (int64_t)seq_q * d_v; }
+    // scores = q . k^T          P(q, k)
+    GemmCall scores(const float *q, const float *k, float *w) const
+    { return GemmCall{0, 1, 0, seq_q, seq_k, d_k, q, d_k, k, d_k, w, seq_k, batch, nq(), nk(), nw()}; }
+    // out = weights . v         P(weights, v)
+    GemmCall context(const float *w, const float *v, float *o) const
+    { return GemmCall{0, 0, 0, seq_q, d_v, seq_k, w, seq_k, v, d_v, o, d_v, batch, nw(), nv(), no()}; }
+    // d(weights) = d(out) . v^T P(d(out), v)
+    GemmCall grad_weights(const float *go, const float *v, float *gw) const
+    { return GemmCall{0, 1, 0, seq_q, seq_k, d_v, go, d_v, v, d_v, gw, seq_k, batch, no(), nv(), nw()}; }
+    // d(v) = weights^T . d(out) P(weights, d(out))
+    GemmCall grad_v(const float *w, const float *go, float *gv) const
+    { return GemmCall{1, 0, 0, seq_k, d_v, seq_q, w, seq_k, go, d_v, gv, d_v, batch, nw(), no(), nv()}; }
+    // d(q) = d(scores) . k      P(d(scores), k)
+    GemmCall grad_q(const float *gs, const float *k, float *gq) const
+    { return GemmCall{0, 0, 0, seq_q, d_k, seq_k, gs, seq_k, k, d_k, gq, d_k, batch, nw(), nk(), nq()}; }
+    // d(k) = (q^T . d(scores))^T = d(scores)^T . q with the LUT fed as P(q, d(scores))
+    GemmCall grad_k(const float *gs, const float *q, float *gk) const
+    { return GemmCall{1, 0, 1, seq_k, d_k, seq_q, gs, seq_k, q, d_k, gk, d_k, batch, nw(), nq(), nk()}; }
+};
+
+bool attn_shape_ok(const AttnShape &s) { return s.batch >= 0 && s.seq_q >= 0 && s.seq_k >= 0 && s.d_k >= 0 && s.d_v >= 0; }
+size_t align256(size_t b) { return (b + 255) / 256 * 256; }
+
+}  // namespace
+
+size_t amsim_attention_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v)
+{
+    const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
+    if (!attn_shape_ok(s)) return 0;
+    return std::max(gemm_ws(s.scores(nullptr, nullptr, nullptr)), gemm_ws(s.context(nullptr, nullptr, nullptr)));
+}
+
+int amsim_attention_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *mask,
+                        int mask_batch_div, int64_t mask_batch_stride, int64_t mask_row_stride, int batch, int seq_q,
+                        int seq_k, int d_k, int d_v, float divisor, float *weights, float *out, void *workspace,
+                        size_t workspace_bytes, void *stream)
+{
+    const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
+    if (!attn_shape_ok(s)) return fail(AMSIM_ERR_INVALID, "negative extent");
+    if (!(divisor > 0.0f)) return fail(AMSIM_ERR_INVALID, "the score divisor must be positive");
+    if (mask && (mask_batch_div < 1 || mask_batch_stride < 0 || mask_row_stride < 0))
+        return fail(AMSIM_ERR_INVALID, "bad mask layout");
+    if (batch == 0 || seq_q == 0) return AMSIM_OK;
+    if (seq_k > 0 && !weights) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    int rc = gemm_call(lut, s.scores(q, k, weights), workspace, workspace_bytes, stream);
+    if (rc != AMSIM_OK) return rc;
+    rc = launch_softmax_rows(weights, mask, mask_batch_div, mask_batch_stride, mask_row_stride, batch, seq_q, seq_k,
+                             divisor, static_cast<hipStream_t>(stream));
+    if (rc != AMSIM_OK) return rc;
+    return gemm_call(lut, s.context(weights, v, out), workspace, workspace_bytes, stream);
+}
+
+size_t amsim_attention_grad_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v)
+{
+    const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
+    if (!attn_shape_ok(s)) return 0;
+    size_t g = gemm_ws(s.grad_weights(nullptr, nullptr, nullptr));
+    g = std::max(g, gemm_ws(s.grad_v(nullptr, nullptr, nullptr)));
+    g = std::max(g, gemm_ws(s.grad_q(nullptr, nullptr, nullptr)));
+    g = std::max(g, gemm_ws(s.grad_k(nullptr, nullptr, nullptr)));
+    return align256((size_t)batch * (size_t)s.nw() * sizeof(float)) + g;
+}
+
+int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *weights,
+                             const float *grad_out, int batch, int seq_q, int seq_k, int d_k, int d_v, float divisor,
+                             float *grad_q, float *grad_k, float *grad_v, void *workspace, size_t workspace_bytes,
+                             void *stream)
+{
+    const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
+    if (!attn_shape_ok(s)) return fail(AMSIM_ERR_INVALID, "negative extent");
+    if (!(divisor > 0.0f)) return fail(AMSIM_ERR_INVALID, "the score divisor must be positive");
+    if (batch == 0) return AMSIM_OK;
+    const size_t need = amsim_attention_grad_workspace_bytes(batch, seq_q, seq_k, d_k, d_v);
+    if (need && (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need))
+        return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
+                                             std::to_string(need) + " bytes");
+    // d(weights), then d(scores) in place, lives at the head of the workspace
+    const size_t gw_bytes = align256((size_t)batch * (size_t)s.nw() * sizeof(float));
+    float *gw = static_cast<float *>(workspace);
+    void *ws = static_cast<uint8_t *>(workspace) + gw_bytes;
+    const size_t ws_bytes = workspace_bytes - gw_bytes;
+    if ((int64_t)seq_q * seq_k > 0 && !weights) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
+    int rc = gemm_call(lut, s.grad_v(weights, grad_out, grad_v), ws, ws_bytes, stream);
+    if (rc != AMSIM_OK) return rc;
+    rc = gemm_call(lut, s.grad_weights(grad_out, v, gw), ws, ws_bytes, stream);
+    if (rc != AMSIM_OK) return rc;
+    rc = launch_softmax_grad_rows(weights, gw, (int64_t)batch * seq_q, seq_k, divisor, static_cast<hipStream_t>(stream));
+    if (rc != AMSIM_OK) return rc;
+    rc = gemm_call(lut, s.grad_q(gw, k, grad_q), ws, ws_bytes, stream);
+    if (rc != AMSIM_OK) return rc;
+    return gemm_call(lut, s.grad_k(gw, q, grad_k), ws, ws_bytes, stream);
+}
+
 // ---- geometry -------------------------------------------------------------------------
 
 int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, int *out_size, int *pad_before)

@@ -116,5 +116,13 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
 
 int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream);
 
+// attention row kernels (in place): scores -> softmax(scores / divisor - 1e9 * mask), and
+// d(weights) -> d(scores); mask element (b, r, j) at mask[(b / batch_div) * batch_stride + r * row_stride + j]
+int launch_softmax_rows(float *scores, const float *mask, int mask_batch_div, int64_t mask_batch_stride,
+                        int64_t mask_row_stride, int64_t batch, int seq_q, int seq_k, float divisor,
+                        hipStream_t stream);
+int launch_softmax_grad_rows(const float *weights, float *grad, int64_t rows, int seq_k, float divisor,
+                             hipStream_t stream);
+
 }  // namespace amsim
 #endif

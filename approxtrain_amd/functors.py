@@ -228,3 +228,85 @@ def matmulam(lut, a, b):
     if out.numel() and ca == 0:
         pass  # an empty reduction yields zeros (matmulam.cc:154-160); the library writes them
     return out
+
+
+def _mask_layout(mask, lead, seq_q, seq_k, device):
+    """Layout of an attention mask broadcastable to ``lead + (seq_q, seq_k)`` for the library:
+    (tensor kept alive, pointer, batch divisor, batch stride, row stride).  A mask shared by the
+    trailing leading dimensions (the heads) and / or by the queries is passed as it is; any
+    other broadcast pattern is materialised."""
+    if mask is None:
+        return None, C.c_void_p(0), 1, 0, 0
+    m = mask.to(device=device, dtype=torch.float32)
+    full = tuple(lead) + (seq_q, seq_k)
+    m = m.reshape((1,) * (len(full) - m.dim()) + tuple(m.shape)) if m.dim() < len(full) else m
+    if m.dim() != len(full) or any(a not in (1, b) for a, b in zip(m.shape, full)):
+        raise ValueError("mask does not broadcast against the attention scores")
+    batch = 1
+    for d in lead:
+        batch *= d
+    rows_shared = m.shape[-2] == 1 and seq_q > 1
+    # leading dimensions: the mask may vary over a prefix of them and be shared by the rest
+    varying = [i for i, d in enumerate(lead) if d > 1 and m.shape[i] == d]
+    shared = [i for i, d in enumerate(lead) if d > 1 and m.shape[i] == 1]
+    prefix_ok = not varying or not shared or max(varying) < min(shared)
+    if m.shape[-1] != seq_k or not prefix_ok:
+        m = m.expand(full).contiguous()
+        return m, _ptr(m), 1, seq_q * seq_k, seq_k
+    div = 1
+    for i in shared:
+        div *= lead[i]
+    m = m.contiguous()
+    row_stride = 0 if rows_shared else seq_k
+    per_item = seq_k if rows_shared else m.shape[-2] * seq_k
+    batch_stride = per_item if varying else 0
+    return m, _ptr(m), div, batch_stride, row_stride
+
+
+def attention(lut, q, k, v, divisor, mask=None):
+    """DotProductAttention.call on ``[..., seq, depth]`` operands with identical leading
+    dimensions: returns (out, weights).  Both products go through the LUT; the division by
+    ``divisor``, the mask term and the softmax are plain FP32."""
+    q, k, v = _dev(q, "queries"), _dev(k, "keys"), _dev(v, "values")
+    lut = _lut(lut)
+    if q.dim() < 2 or q.dim() != k.dim() or q.dim() != v.dim() or q.shape[:-2] != k.shape[:-2] or q.shape[:-2] != v.shape[:-2]:
+        raise ValueError("queries, keys and values need identical leading dimensions")
+    lead = tuple(q.shape[:-2])
+    sq, dk = q.shape[-2:]
+    sk, dk2 = k.shape[-2:]
+    sk2, dv = v.shape[-2:]
+    if dk != dk2 or sk != sk2:
+        raise ValueError("keys must match the queries' depth and the values' length")
+    batch = 1
+    for d in lead:
+        batch *= d
+    keep, mptr, mdiv, mbs, mrs = _mask_layout(mask, lead, sq, sk, q.device)
+    weights = torch.empty(lead + (sq, sk), dtype=torch.float32, device=q.device)
+    out = torch.empty(lead + (sq, dv), dtype=torch.float32, device=q.device)
+    lib = load_library()
+    nbytes = lib.amsim_attention_workspace_bytes(batch, sq, sk, dk, dv)
+    ws, wsp = _workspace(nbytes, q.device)
+    check(lib.amsim_attention_f32(lut.handle, _ptr(q), _ptr(k), _ptr(v), mptr, mdiv, mbs, mrs, batch, sq, sk, dk, dv,
+                                  float(divisor), _ptr(weights), _ptr(out), wsp, nbytes, _stream()))
+    return out, weights
+
+
+def attention_grad(lut, q, k, v, weights, grad_out, divisor):
+    """Gradients of ``attention`` with respect to queries, keys and values."""
+    q, k, v = _dev(q, "queries"), _dev(k, "keys"), _dev(v, "values")
+    weights, grad_out = _dev(weights, "weights"), _dev(grad_out, "grad_out")
+    lut = _lut(lut)
+    lead = tuple(q.shape[:-2])
+    sq, dk = q.shape[-2:]
+    sk, dv = v.shape[-2:]
+    batch = 1
+    for d in lead:
+        batch *= d
+    gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    lib = load_library()
+    nbytes = lib.amsim_attention_grad_workspace_bytes(batch, sq, sk, dk, dv)
+    ws, wsp = _workspace(nbytes, q.device)
+    check(lib.amsim_attention_grad_f32(lut.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(weights), _ptr(grad_out), batch,
+                                       sq, sk, dk, dv, float(divisor), _ptr(gq), _ptr(gk), _ptr(gv), wsp, nbytes,
+                                       _stream()))
+    return gq, gk, gv

@@ -196,20 +196,36 @@ class denseam(nn.Module):
         return {"units": self.units, "use_bias": self.use_bias, "mant_mul_lut": self.mant_mul_lut}
 
 
+class _Attention(torch.autograd.Function):
+    """The whole of DotProductAttention.call as one library call per direction; the mask is a
+    constant (no gradient), as in the reference."""
+
+    @staticmethod
+    def forward(ctx, queries, keys, values, mask, divisor, mant_mul_lut):
+        out, weights = functors.attention(mant_mul_lut, queries, keys, values, divisor, mask)
+        ctx.save_for_backward(queries, keys, values, weights)
+        ctx.attrs = (divisor, mant_mul_lut)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        queries, keys, values, weights = ctx.saved_tensors
+        divisor, lut = ctx.attrs
+        gq, gk, gv = functors.attention_grad(lut, queries, keys, values, weights, grad.contiguous(), divisor)
+        return gq, gk, gv, None, None, None
+
+
 class DotProductAttention(nn.Module):
-    """Scaled dot-product attention with both matrix products through
-    ``matmulam`` (multihead_attention.py:9-30)."""
+    """Scaled dot-product attention with both matrix products through the approximate
+    multiplier (multihead_attention.py:9-30): ``matmulam(softmax(matmulam(q, k^T) / sqrt(d_k)
+    + -1e9 * mask), v)``, run as one strided batch over every leading dimension."""
 
     def __init__(self, lut_file):
         super().__init__()
         self.lut_file = lut_file
 
     def forward(self, queries, keys, values, d_k, mask=None):
-        scores = matmulam(queries, keys, transpose_b=True, mant_mul_lut=self.lut_file) / math.sqrt(float(d_k))
-        if mask is not None:
-            scores = scores + -1e9 * mask
-        weights = torch.softmax(scores, dim=-1)
-        return matmulam(weights, values, mant_mul_lut=self.lut_file)
+        return _Attention.apply(queries, keys, values, mask, math.sqrt(float(d_k)), self.lut_file)
 
 
 class MultiHeadAttention(nn.Module):

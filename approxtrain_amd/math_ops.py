@@ -5,7 +5,8 @@ Differences from the reference, on purpose:
   * transposes are passed to the GEMM as operand strides instead of being
     materialised with ``matrix_transpose`` (math_ops.py:92-93);
   * the gradient passes the LUT on (the reference's gradient calls omit the
-    required ``mant_mul_lut`` attr, math_ops.py:100-156);
+    required ``mant_mul_lut`` attr, math_ops.py:100-156); its LUT operand order
+    is the one the reference's op-level rule gives: (grad, b) and (a, grad);
   * operands of rank > 3 (the (batch, heads, seq, depth) tensors that the
     reference's attention layer feeds, multihead_attention.py:56-57) are
     flattened to a strided batch; the reference's C++ op accepts rank <= 3."""
@@ -39,26 +40,23 @@ class _MatMulAM(torch.autograd.Function):
                 x = x.sum(dim=0, keepdim=like.dim() == 3)
             return x
 
-        # math_ops.py:141-157: the four transpose cases, each a MatMulAM of (first, second) in LUT operand order
+        # The reference's op receives operands that Python has already transposed, with its own
+        # transpose attrs at their default (math_ops.py:92-93), so its gradient always takes the
+        # first branch of math_ops.py:145-147:
+        #     d(a_op) = MatMulAM(grad, b_op^T)        d(b_op) = MatMulAM(a_op^T, grad)
+        # and autodiff transposes d(a_op) / d(b_op) back.  Here the transposes are strides; a
+        # gradient produced transposed keeps its LUT operand order through swap_operands.
         if ctx.needs_input_grad[0]:
-            if not t_a and not t_b:
-                grad_a = g(lut, grad, b, trans_b=True)           # MatMulAM(grad, b^T)
-            elif not t_a and t_b:
-                grad_a = g(lut, grad, b)                          # MatMulAM(grad, b)
-            elif t_a and not t_b:
-                grad_a = g(lut, b, grad, trans_b=True)           # MatMulAM(b, grad^T)
+            if not t_a:
+                grad_a = g(lut, grad, b, trans_b=not t_b)                                  # P(grad, b)
             else:
-                grad_a = g(lut, b, grad, trans_a=True, trans_b=True)  # MatMulAM(b^T, grad^T)
+                grad_a = g(lut, b, grad, trans_a=t_b, trans_b=True, swap_operands=True)    # transposed, still P(grad, b)
             grad_a = unbroadcast(grad_a, a)
         if ctx.needs_input_grad[1]:
-            if not t_a and not t_b:
-                grad_b = g(lut, a, grad, trans_a=True)           # MatMulAM(a^T, grad)
-            elif not t_a and t_b:
-                grad_b = g(lut, grad, a, trans_a=True)           # MatMulAM(grad^T, a)
-            elif t_a and not t_b:
-                grad_b = g(lut, a, grad)                          # MatMulAM(a, grad)
+            if not t_b:
+                grad_b = g(lut, a, grad, trans_a=not t_a)                                  # P(a, grad)
             else:
-                grad_b = g(lut, grad, a, trans_a=True, trans_b=True)  # MatMulAM(grad^T, a^T)
+                grad_b = g(lut, grad, a, trans_a=True, trans_b=t_a, swap_operands=True)    # transposed, still P(a, grad)
             grad_b = unbroadcast(grad_b, b)
         return grad_a, grad_b, None, None, None
 

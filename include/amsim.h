@@ -189,6 +189,36 @@ int amsim_matmulam_f32(amsim_lut_t lut, const float *a, const float *b, int batc
                        int col_a, int row_b, int col_b, float *out, void *workspace, size_t workspace_bytes,
                        void *stream);
 
+/* ---- DotProductAttention.call (ammha/multihead_attention.py:9-30) -------------
+ * for `batch` independent (batch x head) items on contiguous operands
+ * q[batch][seq_q][d_k], k[batch][seq_k][d_k], v[batch][seq_k][d_v]:
+ *   scores  = matmulam(q, k^T) / divisor  [+ -1e9 * mask]     (:18-24)
+ *   weights = softmax(scores) over the key axis                (:27)
+ *   out     = matmulam(weights, v)                             (:30)
+ * Both products go through the LUT (one strided-batch launch each instead of
+ * the per-item loop of cuda/matmulam_kernel.cu:30-98); the division, mask and
+ * softmax are plain FP32 like the TensorFlow ops the reference uses there.
+ * weights[batch][seq_q][seq_k] is an output (the gradient needs it),
+ * out[batch][seq_q][d_v].  mask may be NULL; otherwise its element for item b,
+ * query r, key j is mask[(b / mask_batch_div) * mask_batch_stride +
+ * r * mask_row_stride + j], which covers a mask shared by the heads of one
+ * sample (mask_batch_div = heads) and masks broadcast over queries (row stride 0). */
+size_t amsim_attention_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v);
+int amsim_attention_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *mask,
+                        int mask_batch_div, int64_t mask_batch_stride, int64_t mask_row_stride, int batch, int seq_q,
+                        int seq_k, int d_k, int d_v, float divisor, float *weights, float *out, void *workspace,
+                        size_t workspace_bytes, void *stream);
+/* Gradient of the above with MatMulAM's gradient rule (python/ops/math_ops.py:141-157: the op
+ * never sees the transpose flags, so each product's gradients are matmulam(grad, b_op^T) and
+ * matmulam(a_op^T, grad)):  d(v) = weights^T . d(out),  d(weights) = d(out) . v^T,
+ * d(scores) = softmax gradient / divisor,  d(q) = d(scores) . k,  d(k) = (q^T . d(scores))^T.
+ * The workspace also holds d(scores) (batch * seq_q * seq_k floats). */
+size_t amsim_attention_grad_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v);
+int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *weights,
+                             const float *grad_out, int batch, int seq_q, int seq_k, int d_k, int d_v, float divisor,
+                             float *grad_q, float *grad_k, float *grad_v, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
 /* ---- op-level host logic (what the OpKernel::Compute bodies derive) ----------
  * TensorFlow 2.3 GetWindowedOutputSizeVerbose for dilation 1 as used at
  * convam.cc:382-387, 553-572, 1071-1084: output extent and leading pad. */

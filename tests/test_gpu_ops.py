@@ -89,6 +89,37 @@ def test_matmulam_forward_and_gradient_formulas(ta, tb):
     assert np.array_equal(got.view(np.uint32), cpu.gemm(L, 7, a2, b2, transA=ta, transB=tb).view(np.uint32))
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_matmulam_gradient_operand_order_with_asymmetric_lut(ta, tb, tmp_path):
+    """The reference's op is handed operands that Python already transposed and never sees the
+    flags (math_ops.py:92-93), so its gradients are MatMulAM(grad, b_op^T) and
+    MatMulAM(a_op^T, grad) (math_ops.py:145-147): the LUT is fed (grad, b) and (a, grad) in
+    every transpose case.  An order-sensitive table makes any other order visible."""
+    from approxtrain_amd.math_ops import matmulam
+    from tests.gpu_util import asym_lut_u8
+    tab = asym_lut_u8(3)
+    path = tmp_path / "ASYM_3.bin"
+    path.write_bytes(tab.tobytes())
+    L = cpu.expand_u8(tab, 3)
+    rng = np.random.default_rng(11 + 2 * ta + tb)
+    M, N, K = 37, 21, 45
+    a = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+    b = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    at, bt = dev(a).requires_grad_(True), dev(b).requires_grad_(True)
+    matmulam(at, bt, transpose_a=ta, transpose_b=tb, mant_mul_lut=str(path)).backward(dev(g))
+    a_op = np.ascontiguousarray(a.T if ta else a)
+    b_op = np.ascontiguousarray(b.T if tb else b)
+    ga_op = cpu.gemm(L, 3, g, b_op, transB=True)
+    gb_op = cpu.gemm(L, 3, a_op, g, transA=True)
+    want_a = np.ascontiguousarray(ga_op.T if ta else ga_op)
+    want_b = np.ascontiguousarray(gb_op.T if tb else gb_op)
+    assert np.array_equal(host(at.grad).view(np.uint32), want_a.view(np.uint32))
+    assert np.array_equal(host(bt.grad).view(np.uint32), want_b.view(np.uint32))
+    # and the other order really differs with this table
+    assert not np.array_equal(cpu.gemm(L, 3, g, b_op, transB=True, swap=True).view(np.uint32), ga_op.view(np.uint32))
+
+
 def test_matmulam_rank4_and_broadcast_gradient():
     from approxtrain_amd.math_ops import matmulam
     rng = np.random.default_rng(4)
