@@ -1,0 +1,78 @@
+"""The entry points only enqueue kernels on the caller's stream (no allocation,
+no synchronisation, no memset or copy nodes), so a training step can be captured
+into a HIP graph and replayed.  Every replay is checked against the eager result
+on the same inputs, bit for bit, with eager work and synchronisation between
+replays."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import host
+from tests.util import lut_path
+
+pytestmark = pytest.mark.gpu
+MBM = lut_path("MBM", 7)
+
+
+def _bits(t):
+    return host(t).view(np.uint32)
+
+
+def _step(lut, x, w, dy):
+    from approxtrain_amd import functors
+    y = functors.convam(lut, x, w, (1, 1), "SAME", bias=None, activation=None)
+    dx = functors.convam_input_grad(lut, tuple(x.shape), w, dy, (1, 1), "SAME")
+    dw = functors.convam_filter_grad(lut, x, tuple(w.shape), dy, (1, 1), "SAME")   # splits its reduction
+    return y, dx, dw
+
+
+def test_conv_training_step_replays_from_a_graph():
+    from approxtrain_amd import ApproxMulLut
+    lut = ApproxMulLut.cached(MBM)
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    shape_x, shape_w, shape_y = (4, 28, 28, 32), (3, 3, 32, 48), (4, 28, 28, 48)
+    x, w, dy = (torch.randn(s, device="cuda", generator=gen) for s in (shape_x, shape_w, shape_y))
+    _step(lut, x, w, dy)                       # warm-up outside the capture (plans, LUT upload)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = _step(lut, x, w, dy)
+    for _ in range(3):
+        for t in (x, w, dy):                   # new values in the captured input buffers
+            t.copy_(torch.randn(t.shape, device="cuda", generator=gen))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = _step(lut, x, w, dy)
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert np.array_equal(_bits(got), _bits(want))
+
+
+def test_attention_and_dense_replay_from_a_graph():
+    from approxtrain_amd import ApproxMulLut, functors
+    lut = ApproxMulLut.cached(MBM)
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    q, k, v, go = (torch.randn(6, 64, 32, device="cuda", generator=gen) for _ in range(4))
+    wt = torch.randn(32, 40, device="cuda", generator=gen)
+    bias = torch.randn(40, device="cuda", generator=gen)
+
+    def step():
+        out, wts = functors.attention(lut, q, k, v, 5.0)
+        grads = functors.attention_grad(lut, q, k, v, wts, go, 5.0)
+        proj = functors.denseam(lut, out.reshape(-1, 32), wt, bias=bias, activation="relu")
+        return (out, wts, proj) + tuple(grads)
+
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for _ in range(3):
+        for t in (q, k, v, go):
+            t.copy_(torch.randn(t.shape, device="cuda", generator=gen))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = step()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert np.array_equal(_bits(got), _bits(want))
