@@ -461,6 +461,20 @@ void lutgemm_kernel(KArgs a)
                 const uint32_t chan = (uint32_t)rl;
                 const int64_t kleft64 = a.K - kfirst;
                 const int kleft = kleft64 < ELEMS ? (int)kleft64 : ELEMS;  // elements of this run inside K
+                if (a.p.GW % ELEMS == 0) {
+                    // runs start at multiples of ELEMS, so one never leaves its output row: (b, y)
+                    // and the source row are fixed, only the column advances
+                    const bool row_ok = (unsigned)iy < (unsigned)a.p.SH;
+#pragma unroll
+                    for (int i = 0; i < ELEMS; ++i) {
+                        uint32_t v = 0;
+                        if (i < kleft && row_ok && (unsigned)ix < (unsigned)a.p.SW) v = f2u((pbase + soff)[chan]);
+                        pv[i] = v;
+                        sr.add(v);
+                        ix += a.p.sx;
+                        soff += step;
+                    }
+                } else
 #pragma unroll
                 for (int i = 0; i < ELEMS; ++i) {
                     uint32_t v = 0;
