@@ -15,13 +15,125 @@ from .amnn_ops import amconvolution_v2
 from .math_ops import matmulam
 
 
+# Keras vocabulary of the reference's layers (activations.get / initializers.get,
+# am_convolutional.py:128-144, amdenselayer.py:109-126): names map to torch functions.
+_ACTIVATIONS = {
+    "linear": None,
+    "relu": torch.relu,
+    "sigmoid": torch.sigmoid,
+    "tanh": torch.tanh,
+    "softmax": lambda x: torch.softmax(x, dim=-1),
+    "softplus": nn.functional.softplus,
+    "softsign": nn.functional.softsign,
+    "elu": nn.functional.elu,
+    "selu": nn.functional.selu,
+    "gelu": nn.functional.gelu,
+    "swish": nn.functional.silu,
+    "exponential": torch.exp,
+}
+
+
+def _get_activation(activation):
+    """None, a Keras activation name, or a callable -> callable or None (identity)."""
+    if activation is None or callable(activation):
+        return activation
+    if isinstance(activation, str) and activation in _ACTIVATIONS:
+        return _ACTIVATIONS[activation]
+    raise ValueError(f"Unknown activation function: {activation}")
+
+
 def _fusable(activation):
     """Name of the activation if the library can apply it in the producing kernel, else None."""
     if activation is None:
         return "linear"
-    if activation in ("relu", torch.relu, torch.nn.functional.relu) or isinstance(activation, nn.ReLU):
+    if activation in (torch.relu, torch.nn.functional.relu) or isinstance(activation, nn.ReLU):
         return "relu"
     return None
+
+
+def _initialize_(t, initializer, fan_in, fan_out):
+    """Fills ``t`` in place by a Keras initializer name, or by a callable ``f(shape)`` that
+    returns the values."""
+    with torch.no_grad():
+        if callable(initializer):
+            return t.copy_(torch.as_tensor(initializer(tuple(t.shape)), dtype=t.dtype))
+        name = str(initializer).lower()
+        if name == "zeros":
+            return t.zero_()
+        if name == "ones":
+            return t.fill_(1.0)
+        if name == "random_normal":
+            return t.normal_(0.0, 0.05)
+        if name == "random_uniform":
+            return t.uniform_(-0.05, 0.05)
+        scale = {"glorot": 2.0 / (fan_in + fan_out), "he": 2.0 / fan_in, "lecun": 1.0 / fan_in}
+        for family, variance in scale.items():
+            if name == family + "_uniform":
+                limit = math.sqrt(3.0 * variance)
+                return t.uniform_(-limit, limit)
+            if name == family + "_normal":
+                # Keras draws from a normal truncated at two standard deviations and rescales
+                std = math.sqrt(variance) / 0.87962566103423978
+                return nn.init.trunc_normal_(t, 0.0, std, -2.0 * std, 2.0 * std)
+        raise ValueError(f"Unknown initializer: {initializer}")
+
+
+class _KerasLayerArgs:
+    """Constructor arguments every Keras layer of the reference accepts besides its own:
+    regularizers and constraints are kept as callables (``losses()`` evaluates the
+    regularizers, ``apply_constraints()`` projects the parameters); ``name``, ``dtype``,
+    ``trainable`` and ``input_shape`` are honoured where they mean something here."""
+
+    def _keras_args(self, kernel_regularizer, bias_regularizer, activity_regularizer, kernel_constraint,
+                    bias_constraint, kwargs):
+        for what, f in (("kernel_regularizer", kernel_regularizer), ("bias_regularizer", bias_regularizer),
+                        ("activity_regularizer", activity_regularizer), ("kernel_constraint", kernel_constraint),
+                        ("bias_constraint", bias_constraint)):
+            if f is not None and not callable(f):
+                raise ValueError(f"{what} must be a callable or None")
+        self.kernel_regularizer, self.bias_regularizer = kernel_regularizer, bias_regularizer
+        self.activity_regularizer = activity_regularizer
+        self.kernel_constraint, self.bias_constraint = kernel_constraint, bias_constraint
+        self.layer_name = kwargs.pop("name", None)
+        self.trainable = bool(kwargs.pop("trainable", True))
+        dtype = kwargs.pop("dtype", None)
+        if dtype not in (None, "float32", torch.float32):
+            raise ValueError("the approximate-multiplier ops are float32 only")
+        input_shape = kwargs.pop("input_shape", None)
+        kwargs.pop("batch_input_shape", None)
+        if kwargs:
+            raise TypeError(f"Keyword argument not understood: {sorted(kwargs)[0]}")
+        self._activity_loss = None
+        return input_shape
+
+    def _finish_build(self):
+        if not self.trainable:
+            for p in self.parameters():
+                p.requires_grad_(False)
+
+    def _track_activity(self, out):
+        if self.activity_regularizer is not None:
+            self._activity_loss = self.activity_regularizer(out)
+        return out
+
+    def losses(self):
+        """Regularization terms of this layer (Keras ``layer.losses``), to be added to the objective."""
+        out = []
+        if self.kernel_regularizer is not None and self.kernel is not None:
+            out.append(self.kernel_regularizer(self.kernel))
+        if self.bias_regularizer is not None and self.bias is not None:
+            out.append(self.bias_regularizer(self.bias))
+        if self._activity_loss is not None:
+            out.append(self._activity_loss)
+        return out
+
+    def apply_constraints(self):
+        """Projects kernel and bias through their constraints (Keras does so after each update)."""
+        with torch.no_grad():
+            if self.kernel_constraint is not None and self.kernel is not None:
+                self.kernel.copy_(self.kernel_constraint(self.kernel))
+            if self.bias_constraint is not None and self.bias is not None:
+                self.bias.copy_(self.bias_constraint(self.bias))
 
 
 def _epilogue_backward(grad, out, bias, act):
@@ -58,46 +170,66 @@ class _ConvamBiasAct(torch.autograd.Function):
         return grad_input, grad_filter, grad_bias, None, None, None, None
 
 
-def _glorot_uniform_(t, fan_in, fan_out):
-    limit = math.sqrt(6.0 / (fan_in + fan_out))
-    with torch.no_grad():
-        return t.uniform_(-limit, limit)
-
-
-class AMConv2D(nn.Module):
+class AMConv2D(nn.Module, _KerasLayerArgs):
     """2-D convolution over NHWC input with an HWIO kernel through op ``Convam``.
-    Same constructor vocabulary as the Keras layer: ``filters, kernel_size,
-    strides, padding ('valid' | 'same'), activation, use_bias, mant_mul_lut``."""
+    Same constructor vocabulary as the Keras layer (am_convolutional.py:519-558):
+    ``filters, kernel_size, strides, padding ('valid' | 'same'), data_format, dilation_rate,
+    groups, activation, use_bias, kernel_initializer, bias_initializer, the regularizers and
+    constraints, mant_mul_lut``.  Like the reference, only channels-last data, dilation 1
+    (amnn_ops.py:196-197) and one group run through the approximate op."""
 
-    def __init__(self, filters, kernel_size, strides=(1, 1), padding="valid", activation=None, use_bias=True,
-                 mant_mul_lut='', in_channels=None, dilation_rate=(1, 1)):
+    def __init__(self, filters, kernel_size, strides=(1, 1), padding="valid", data_format=None,
+                 dilation_rate=(1, 1), groups=1, activation=None, use_bias=True,
+                 kernel_initializer="glorot_uniform", bias_initializer="zeros", kernel_regularizer=None,
+                 bias_regularizer=None, activity_regularizer=None, kernel_constraint=None, bias_constraint=None,
+                 mant_mul_lut='', in_channels=None, **kwargs):
         super().__init__()
         if not mant_mul_lut:
             raise ValueError("mant_mul_lut must name a LUT file")
         ks = (kernel_size, kernel_size) if isinstance(kernel_size, int) else tuple(kernel_size)
         st = (strides, strides) if isinstance(strides, int) else tuple(strides)
         dr = (dilation_rate, dilation_rate) if isinstance(dilation_rate, int) else tuple(dilation_rate)
+        if len(ks) != 2 or len(st) != 2 or len(dr) != 2:
+            raise ValueError("kernel_size, strides and dilation_rate take one or two integers")
+        if filters is not None and int(filters) < 0:
+            raise ValueError(f"Received a negative value for `filters`. Was expecting a positive value, got {filters}.")
         if any(d != 1 for d in dr):
             raise ValueError("Dilation is not supported in current implementation")
+        if padding.lower() == "causal":
+            raise ValueError("Causal padding is only supported for `Conv1D` and `SeparableConv1D`.")
         if padding.lower() not in ("valid", "same"):
             raise ValueError("padding must be 'valid' or 'same'")
+        if data_format not in (None, "channels_last"):
+            raise ValueError("only channels_last (NHWC) data runs through the approximate convolution")
+        if groups != 1:
+            raise ValueError("grouped convolution is not provided by the approximate convolution op")
         self.filters, self.kernel_size, self.strides = int(filters), ks, st
         self.padding = padding.upper()
-        self.activation, self.use_bias, self.mant_mul_lut = activation, use_bias, mant_mul_lut
+        self.activation, self.use_bias, self.mant_mul_lut = _get_activation(activation), use_bias, mant_mul_lut
+        self.kernel_initializer, self.bias_initializer = kernel_initializer, bias_initializer
+        input_shape = self._keras_args(kernel_regularizer, bias_regularizer, activity_regularizer, kernel_constraint,
+                                       bias_constraint, kwargs)
         self.kernel = None
         self.bias = None
+        if in_channels is None and input_shape is not None:
+            in_channels = input_shape[-1]
         if in_channels is not None:
             self.build(in_channels)
 
     def build(self, in_channels, device=None):
         kh, kw = self.kernel_size
         k = torch.empty(kh, kw, in_channels, self.filters, device=device)
-        _glorot_uniform_(k, kh * kw * in_channels, kh * kw * self.filters)
+        _initialize_(k, self.kernel_initializer, kh * kw * in_channels, kh * kw * self.filters)
         self.kernel = nn.Parameter(k)
         if self.use_bias:
-            self.bias = nn.Parameter(torch.zeros(self.filters, device=device))
+            b = torch.empty(self.filters, device=device)
+            self.bias = nn.Parameter(_initialize_(b, self.bias_initializer, self.filters, self.filters))
+        self._finish_build()
 
     def forward(self, inputs):
+        return self._track_activity(self._call(inputs))
+
+    def _call(self, inputs):
         if self.kernel is None:
             self.build(inputs.shape[-1], inputs.device)
         act = _fusable(self.activation)
@@ -154,30 +286,45 @@ class _DenseamBiasAct(torch.autograd.Function):
         return grad_input, grad_weights, grad_bias, None, None
 
 
-class denseam(nn.Module):
-    """Dense layer through op ``Denseam``: ``activation(inputs . kernel + bias)``.
-    Inputs of rank > 2 are flattened to [-1, width] and go through the same op
-    (the reference routes them to an exact ``tensordot``, amdenselayer.py:215,
-    which silently bypasses the approximate multiplier)."""
+class denseam(nn.Module, _KerasLayerArgs):
+    """Dense layer through op ``Denseam``: ``activation(inputs . kernel + bias)``, with the Keras
+    constructor vocabulary of amdenselayer.py:93-126.  Inputs of rank > 2 are flattened to
+    [-1, width] and go through the same op (the reference routes them to an exact
+    ``tensordot``, amdenselayer.py:215, which silently bypasses the approximate multiplier)."""
 
-    def __init__(self, units, activation=None, use_bias=True, mant_mul_lut='', input_dim=None):
+    def __init__(self, units, activation=None, use_bias=True, kernel_initializer="glorot_uniform",
+                 bias_initializer="zeros", kernel_regularizer=None, bias_regularizer=None, activity_regularizer=None,
+                 kernel_constraint=None, bias_constraint=None, mant_mul_lut='', input_dim=None, **kwargs):
         super().__init__()
         if not mant_mul_lut:
             raise ValueError("mant_mul_lut must name a LUT file")
-        self.units, self.activation, self.use_bias, self.mant_mul_lut = int(units), activation, use_bias, mant_mul_lut
+        if int(units) < 0:
+            raise ValueError(f"Received an invalid value for `units`, expected a positive integer, got {units}.")
+        self.units, self.use_bias, self.mant_mul_lut = int(units), use_bias, mant_mul_lut
+        self.activation = _get_activation(activation)
+        self.kernel_initializer, self.bias_initializer = kernel_initializer, bias_initializer
+        input_shape = self._keras_args(kernel_regularizer, bias_regularizer, activity_regularizer, kernel_constraint,
+                                       bias_constraint, kwargs)
         self.kernel = None
         self.bias = None
+        if input_dim is None and input_shape is not None:
+            input_dim = input_shape[-1]
         if input_dim is not None:
             self.build(input_dim)
 
     def build(self, input_dim, device=None):
         k = torch.empty(input_dim, self.units, device=device)
-        _glorot_uniform_(k, input_dim, self.units)
+        _initialize_(k, self.kernel_initializer, input_dim, self.units)
         self.kernel = nn.Parameter(k)
         if self.use_bias:
-            self.bias = nn.Parameter(torch.zeros(self.units, device=device))
+            b = torch.empty(self.units, device=device)
+            self.bias = nn.Parameter(_initialize_(b, self.bias_initializer, self.units, self.units))
+        self._finish_build()
 
     def forward(self, inputs):
+        return self._track_activity(self._call(inputs))
+
+    def _call(self, inputs):
         if self.kernel is None:
             self.build(inputs.shape[-1], inputs.device)
         lead = inputs.shape[:-1]

@@ -142,3 +142,37 @@ def test_layers_validate_constructor_arguments():
     assert tuple(layer.kernel.shape) == (5, 5, 1, 6) and layer.get_config()["mant_mul_lut"] == "MBM_7.bin"
     d = denseam(300, mant_mul_lut="MBM_7.bin", input_dim=784)
     assert tuple(d.kernel.shape) == (784, 300)
+
+
+def test_layers_take_the_keras_constructor_vocabulary():
+    """am_convolutional.py:519-558 / amdenselayer.py:93-126: initializers and activations by
+    name, regularizers, constraints, name / input_shape / trainable; what the approximate op
+    cannot do is refused with a message (channels_first, groups, causal padding)."""
+    import math
+    from approxtrain_amd.layers import AMConv2D, denseam
+    lut = "MBM_7.bin"
+    torch.manual_seed(0)
+    c = AMConv2D(64, (3, 3), strides=2, padding="same", data_format="channels_last", activation="relu",
+                 kernel_initializer="he_normal", bias_initializer="ones", kernel_regularizer=lambda w: (w * w).sum(),
+                 kernel_constraint=lambda w: w.clamp(-0.01, 0.01), mant_mul_lut=lut, input_shape=(56, 56, 64), name="conv")
+    assert tuple(c.kernel.shape) == (3, 3, 64, 64) and c.layer_name == "conv" and c.activation is torch.relu
+    assert abs(float(c.kernel.detach().std()) - math.sqrt(2.0 / 576)) < 0.1 * math.sqrt(2.0 / 576)
+    assert float(c.kernel.detach().abs().max()) <= 2.0 * math.sqrt(2.0 / 576) / 0.8796 + 1e-6   # truncated at two sigma
+    assert torch.equal(c.bias.detach(), torch.ones(64))
+    assert len(c.losses()) == 1 and float(c.losses()[0].detach()) == pytest.approx(float((c.kernel.detach() ** 2).sum()))
+    c.apply_constraints()
+    assert float(c.kernel.detach().abs().max()) <= 0.01
+    d = denseam(10, activation="softmax", kernel_initializer="glorot_uniform", bias_regularizer=lambda b: b.abs().sum(),
+                mant_mul_lut=lut, input_dim=300, trainable=False)
+    assert float(d.kernel.detach().abs().max()) <= math.sqrt(6.0 / 310) and not d.kernel.requires_grad
+    assert callable(d.activation) and torch.allclose(d.activation(torch.zeros(2, 4)), torch.full((2, 4), 0.25))
+    custom = denseam(3, kernel_initializer=lambda shape: torch.full(shape, 0.5), mant_mul_lut=lut, input_dim=2)
+    assert torch.equal(custom.kernel.detach(), torch.full((2, 3), 0.5))
+    for bad in (dict(data_format="channels_first"), dict(groups=2), dict(padding="causal"), dict(activation="nope"),
+                dict(kernel_initializer="nope", in_channels=3), dict(kernel_regularizer=0.1), dict(dtype="float16")):
+        with pytest.raises(ValueError):
+            AMConv2D(8, 3, mant_mul_lut=lut, **bad)
+    with pytest.raises(TypeError, match="not understood"):
+        AMConv2D(8, 3, mant_mul_lut=lut, kernel_size2=3)
+    with pytest.raises(ValueError):
+        denseam(8, activation="nope", mant_mul_lut=lut)
