@@ -33,6 +33,33 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert sorted(_lib.SIGNATURES) == names
 
 
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """include/amsim.h must be usable from C (the boundary is a C ABI, not a C++ one): a C99
+    program that includes it compiles without warnings, links against libamsim.so and can call
+    an entry point that needs no device."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_amsim.c"
+    src.write_text(
+        '#include <stdio.h>\n#include "amsim.h"\n'
+        "int main(void) {\n"
+        "  int out = 0, pad = 0;\n"
+        "  if (amsim_conv_geometry(56, 3, 1, AMSIM_PADDING_SAME, &out, &pad) != AMSIM_OK) return 1;\n"
+        "  if (amsim_lut_mant_width((amsim_lut_t)0) != -1) return 2;\n"
+        "  if (amsim_conv_geometry(56, 3, 1, 99, &out, &pad) == AMSIM_OK) return 3;\n"
+        '  printf("%d %d %s\\n", out, pad, amsim_last_error());\n'
+        "  return 0;\n}\n")
+    exe = tmp_path / "use_amsim"
+    libdir = os.path.dirname(_lib.lib_path())
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-L", libdir, "-lamsim", "-Wl,-rpath," + libdir, "-o", str(exe)], check=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert run.returncode == 0, run.stderr
+    assert run.stdout.startswith("56 1 padding must be")
+
+
 def test_tensorflow_bridge_uses_only_declared_entry_points():
     """The TensorFlow bridge cannot be compiled here (no TensorFlow); at least every C-ABI
     call in it must name an entry point the header declares, and every GPU functor of the
