@@ -60,6 +60,32 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
     assert run.stdout.startswith("56 1 padding must be")
 
 
+@pytest.mark.parametrize("mask_shape", [(2, 1, 1, 7), (5, 7), (1, 7), (2, 1, 5, 7), (2, 3, 5, 7), (1, 3, 1, 7),
+                                        (2, 3, 1, 7), (1, 1, 5, 1), (7,)])
+def test_attention_mask_layout_addresses_the_broadcast_mask(mask_shape):
+    """The (divisor, batch stride, row stride) triple handed to the library must address exactly
+    the element that numpy broadcasting picks, for every (item, query, key)."""
+    import numpy as np
+    from approxtrain_amd.functors import _mask_layout
+    lead, sq, sk = (2, 3), 5, 7
+    mask = torch.arange(int(np.prod(mask_shape)), dtype=torch.float32).reshape(mask_shape) + 1.0
+    keep, _, div, bstride, rstride = _mask_layout(mask, lead, sq, sk, torch.device("cpu"))
+    flat = keep.reshape(-1).numpy()
+    want = np.broadcast_to(mask.numpy(), lead + (sq, sk)).reshape(-1, sq, sk)
+    for b in range(want.shape[0]):
+        for r in range(sq):
+            base = (b // div) * bstride + r * rstride
+            assert np.array_equal(flat[base:base + sk], want[b, r]), (b, r)
+
+
+def test_attention_mask_layout_rejects_shapes_that_do_not_broadcast():
+    from approxtrain_amd.functors import _mask_layout
+    with pytest.raises(ValueError):
+        _mask_layout(torch.zeros(2, 4, 7), (2, 3), 5, 7, torch.device("cpu"))
+    with pytest.raises(ValueError):
+        _mask_layout(torch.zeros(2, 3, 5, 7, 1), (2, 3), 5, 7, torch.device("cpu"))
+
+
 def test_tensorflow_bridge_uses_only_declared_entry_points():
     """The TensorFlow bridge cannot be compiled here (no TensorFlow); at least every C-ABI
     call in it must name an entry point the header declares, and every GPU functor of the
