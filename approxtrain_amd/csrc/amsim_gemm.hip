@@ -263,9 +263,21 @@ void lutgemm_kernel(KArgs a)
     const bool active = j0 < a.J;
     const int m = a.m;
 
-    if (!LUTG)
-        for (int i = tid * 16; i < a.lut_bytes; i += WG_THREADS * 16)
-            *reinterpret_cast<uint4 *>(lut_s + i) = *reinterpret_cast<const uint4 *>(a.lut_img + i);
+    if (!LUTG) {
+        // The LUT image goes from global memory straight into LDS, 16 bytes per lane and
+        // instruction, without passing through registers: the copies are only started here and
+        // are waited for together with the first chunk's reads, so a workgroup's start costs
+        // one memory latency instead of one per round of the copy.
+        constexpr int NVEC = LUT_LDS_BYTES / 16;
+#pragma unroll
+        for (int i = 0; i * WG_THREADS < NVEC; ++i) {
+            const int v0 = i * WG_THREADS + wave * 64;  // first vector of this wave's 1 KB slice
+#if defined(__HIP_DEVICE_COMPILE__)  // the builtin exists in the device pass only
+            if ((v0 + lane) * 16 < a.lut_bytes)
+                __builtin_amdgcn_global_load_lds(a.lut_img + (v0 + lane) * 16, lut_s + v0 * 16, 16, 0, 0);
+#endif
+        }
+    }
     if (PK != P_DENSE) fill_rowinfo(a.p, a.R, row0, ROWS, rowinfo);
     if (tid < 2) pflag[tid] = 0u;
     __syncthreads();
@@ -544,6 +556,9 @@ void lutgemm_kernel(KArgs a)
 
     int unsafe = 0;
     if (ch_begin < ch_end) unsafe = load_chunk(ch_begin);
+    // the LUT copies started above have landed in LDS once the vector-memory counter drains;
+    // the barriers at the top of the first trip then order them against every wave's gathers
+    if (!LUTG) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const int lrow = wr * 64 + lane;
     const int mshift = 23 - m;
 
