@@ -224,6 +224,10 @@ struct GradInputGeometry {
     int stride_rows, stride_cols, pad_top, pad_left;
 };
 
+// floats per residue class (a multiple of 64, so every class's vector is 256-byte aligned)
+int poison_stride(int in_depth) { return (in_depth + 63) / 64 * 64; }
+size_t poison_bytes(int in_depth) { return (size_t)MAX_TAP_CLASSES * poison_stride(in_depth) * sizeof(float); }
+
 GemmDesc grad_input_phase(const GradInputGeometry &g, int py, int px, const float *grad, const float *filter,
                           float *output)
 {
@@ -256,8 +260,10 @@ size_t amsim_convam_input_grad_workspace_bytes(int batch, int input_rows, int in
 {
     // The strides are not part of the query (as they are not part of the reference's temporaries'
     // shapes): a strided call runs smaller sub-problems than this stride-1 bound in every extent.
-    return gemm_workspace_bytes((int64_t)batch * input_rows * input_cols, in_depth,
-                                (int64_t)filter_rows * filter_cols * out_depth, 1, 1);
+    // A strided call also keeps one vector of in_depth floats per residue class, for up to
+    // MAX_TAP_CLASSES classes at a time, ahead of the GEMM's own workspace.
+    return poison_bytes(in_depth) + gemm_workspace_bytes((int64_t)batch * input_rows * input_cols, in_depth,
+                                                         (int64_t)filter_rows * filter_cols * out_depth, 1, 1);
 }
 
 size_t amsim_convam_input_grad_strided_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
@@ -272,7 +278,7 @@ size_t amsim_convam_input_grad_strided_workspace_bytes(int batch, int input_rows
     for (int py = 0; py < stride_rows; ++py)
         for (int px = 0; px < stride_cols; ++px) {
             const GemmDesc d = grad_input_phase(g, py, px, nullptr, nullptr, nullptr);
-            need = std::max(need, gemm_workspace_bytes(d.R, d.J, d.K, 1, 1));
+            need = std::max(need, poison_bytes(in_depth) + gemm_workspace_bytes(d.R, d.J, d.K, 1, 1));
         }
     return need;
 }
@@ -303,17 +309,48 @@ int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_gra
                                              std::to_string(need) + " bytes");
     const GradInputGeometry g{batch, input_rows, input_cols, in_depth, filter_rows, filter_cols, out_depth,
                               out_rows, out_cols, stride_rows, stride_cols, pad_top, pad_left};
-    for (int py = 0; py < stride_rows; ++py)
-        for (int px = 0; px < stride_cols; ++px) {
-            GemmDesc d = grad_input_phase(g, py, px, grad, filter, output);
-            if (d.R == 0) continue;
-            // a phase whose best plan wants more partial-sum space than the caller's (stride-agnostic)
-            // workspace holds runs unsplit: its pre-decoded filter always fits
-            if (gemm_workspace_bytes(d.R, d.J, d.K, 1, 1) > workspace_bytes) d.no_split = true;
-            const int rc = run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    float *poison = static_cast<float *>(workspace);
+    void *gemm_ws_ptr = static_cast<uint8_t *>(workspace) + poison_bytes(in_depth);
+    const size_t gemm_ws_bytes = workspace_bytes - poison_bytes(in_depth);
+    const bool strided = stride_rows > 1 || stride_cols > 1;
+    // residue classes with pixels, handled MAX_TAP_CLASSES at a time: one launch marks the channels
+    // that a class's skipped taps poison, then the class's sub-problems run
+    struct Pending { int py, px; };
+    Pending pend[MAX_TAP_CLASSES];
+    TapClass cls[MAX_TAP_CLASSES];
+    int n = 0;
+    auto flush = [&]() -> int {
+        if (n == 0) return AMSIM_OK;
+        if (strided) {
+            const int rc = launch_skipped_tap_poison(filter, filter_rows, filter_cols, in_depth, out_depth, cls, n,
+                                                     poison, poison_stride(in_depth), st);
             if (rc != AMSIM_OK) return rc;
         }
-    return AMSIM_OK;
+        for (int i = 0; i < n; ++i) {
+            GemmDesc d = grad_input_phase(g, pend[i].py, pend[i].px, grad, filter, output);
+            if (strided) d.bias_j = poison + (size_t)i * poison_stride(in_depth);
+            // a phase whose best plan wants more partial-sum space than the caller's (stride-agnostic)
+            // workspace holds runs unsplit: its pre-decoded filter always fits
+            if (gemm_workspace_bytes(d.R, d.J, d.K, 1, 1) > gemm_ws_bytes) d.no_split = true;
+            const int rc = run_gemm(lut->l, d, gemm_ws_ptr, gemm_ws_bytes, st);
+            if (rc != AMSIM_OK) return rc;
+        }
+        n = 0;
+        return AMSIM_OK;
+    };
+    for (int py = 0; py < stride_rows; ++py)
+        for (int px = 0; px < stride_cols; ++px) {
+            const GemmDesc d = grad_input_phase(g, py, px, grad, filter, output);
+            if (d.R == 0) continue;
+            pend[n] = Pending{py, px};
+            cls[n] = TapClass{d.q.fy0, d.q.fsy, d.q.TH, d.q.fx0, d.q.fsx, d.q.TW};
+            if (++n == MAX_TAP_CLASSES) {
+                const int rc = flush();
+                if (rc != AMSIM_OK) return rc;
+            }
+        }
+    return flush();
 }
 
 namespace {

@@ -48,7 +48,6 @@ constexpr int LUT_LDS_BYTES = 16384 + 128;   // 2^(2m) entries + one all-zero ro
 constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels are compiled for
 constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
 constexpr int DEVICE_CUS = 256;               // MI355X; only steers work splitting, never correctness
-constexpr int WG_SLOTS = DEVICE_CUS * WAVES_PER_SIMD;  // workgroups resident at once
 
 static std::atomic<int> g_split_k{1};
 
@@ -271,8 +270,8 @@ void lutgemm_kernel(KArgs a)
         constexpr int NVEC = LUT_LDS_BYTES / 16;
 #pragma unroll
         for (int i = 0; i * WG_THREADS < NVEC; ++i) {
-            const int v0 = i * WG_THREADS + wave * 64;  // first vector of this wave's 1 KB slice
 #if defined(__HIP_DEVICE_COMPILE__)  // the builtin exists in the device pass only
+            const int v0 = i * WG_THREADS + wave * 64;  // first vector of this wave's 1 KB slice
             if ((v0 + lane) * 16 < a.lut_bytes)
                 __builtin_amdgcn_global_load_lds(a.lut_img + (v0 + lane) * 16, lut_s + v0 * 16, 16, 0, 0);
 #endif
@@ -738,6 +737,50 @@ __global__ __launch_bounds__(WG_THREADS) void fill_empty_kernel(RArgs a)
     const int64_t r = idx / a.J, j = idx - r * a.J;
     a.out[(int64_t)blockIdx.y * a.out_batch_stride + out_row_offset(a.ep.omap, a.row_base + r, a.so_r) + j * a.so_j] =
         apply_epilogue(a.ep, 0.0f, a.row_base + r, j);
+}
+
+struct PoisonArgs {
+    const float *filter;
+    int KH, KW, IC, OC, n_classes, out_stride;
+    float *out;
+    TapClass cls[MAX_TAP_CLASSES];
+};
+
+// One wavefront per (class, input channel): lanes run over the output channels of each skipped tap.
+__global__ __launch_bounds__(WG_THREADS) void skipped_tap_poison_kernel(PoisonArgs a)
+{
+    const int lane = threadIdx.x & 63;
+    const int ic = blockIdx.x * (WG_THREADS / 64) + (threadIdx.x >> 6);
+    if (ic >= a.IC) return;
+    const TapClass c = a.cls[blockIdx.y];
+    int bad = 0;
+    for (int fy = 0; fy < a.KH; ++fy)
+        for (int fx = 0; fx < a.KW; ++fx) {
+            // flipped-filter indices, as the sub-problem's operand decoder walks them
+            const int gy = a.KH - 1 - fy, gx = a.KW - 1 - fx;
+            const bool own_y = gy >= c.fy0 && (gy - c.fy0) % c.fsy == 0 && (gy - c.fy0) / c.fsy < c.th;
+            const bool own_x = gx >= c.fx0 && (gx - c.fx0) % c.fsx == 0 && (gx - c.fx0) / c.fsx < c.tw;
+            if (own_y && own_x) continue;
+            const float *w = a.filter + ((int64_t)(fy * a.KW + fx) * a.IC + ic) * a.OC;
+            for (int oc = lane; oc < a.OC; oc += 64) bad |= ((f2u(w[oc]) & 0x7f800000u) == 0x7f800000u) ? 1 : 0;
+        }
+    bad = __any(bad);
+    if (lane == 0) a.out[(int64_t)blockIdx.y * a.out_stride + ic] = bad ? u2f(0x7fc00000u) : 0.0f;
+}
+
+int launch_skipped_tap_poison(const float *filter, int KH, int KW, int IC, int OC, const TapClass *classes,
+                              int n_classes, float *out, int out_stride, hipStream_t stream)
+{
+    if (n_classes <= 0 || IC <= 0) return AMSIM_OK;
+    if (n_classes > MAX_TAP_CLASSES) return fail(AMSIM_ERR_INVALID, "too many tap classes for one launch");
+    PoisonArgs a{};
+    a.filter = filter; a.KH = KH; a.KW = KW; a.IC = IC; a.OC = OC; a.n_classes = n_classes; a.out_stride = out_stride;
+    a.out = out;
+    for (int i = 0; i < n_classes; ++i) a.cls[i] = classes[i];
+    const int per_wg = WG_THREADS / 64;
+    skipped_tap_poison_kernel<<<dim3((unsigned)((IC + per_wg - 1) / per_wg), (unsigned)n_classes), WG_THREADS, 0, stream>>>(a);
+    AMSIM_HIP_CHECK(hipGetLastError());
+    return AMSIM_OK;
 }
 
 static void launch_reduce(const RArgs &ra, hipStream_t stream)

@@ -116,6 +116,19 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
 
 int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream);
 
+// Strided grad-input runs one sub-problem per residue class of the input pixels, each over the
+// filter taps that meet gradient samples.  The reference multiplies the other taps too, with the
+// zeros it inserted between the samples: harmless (+0) unless such a weight is inf or NaN, when
+// 0 x w = NaN reaches every pixel of the class.  This kernel writes, per class and input channel,
+// NaN if a skipped tap holds a non-finite weight and +0 otherwise; the sub-problem adds it as a
+// bias.  A class's own taps are flipped-filter indices f0 + t * stride, t < taps, on each axis.
+struct TapClass {
+    int fy0, fsy, th, fx0, fsx, tw;
+};
+constexpr int MAX_TAP_CLASSES = 16;  // classes handled by one launch
+int launch_skipped_tap_poison(const float *filter, int KH, int KW, int IC, int OC, const TapClass *classes,
+                              int n_classes, float *out, int out_stride, hipStream_t stream);
+
 // attention row kernels (in place): scores -> softmax(scores / divisor - 1e9 * mask), and
 // d(weights) -> d(scores); mask element (b, r, j) at mask[(b / batch_div) * batch_stride + r * row_stride + j]
 int launch_softmax_rows(float *scores, const float *mask, int mask_batch_div, int64_t mask_batch_stride,

@@ -192,3 +192,29 @@ def test_strided_grad_input_with_the_stride_agnostic_workspace():
     sum_abs = np.abs(want).max() * 50 + 1.0
     for got in outs:
         assert np.all(np.abs(got - want) <= 1e-5 * sum_abs)
+
+
+@pytest.mark.parametrize("xs,ws,stride,padding,bad", [
+    ((2, 9, 8, 5), (3, 3, 5, 4), (2, 2), "SAME", np.inf),
+    ((1, 12, 7, 3), (3, 5, 3, 6), (3, 2), "VALID", np.nan),
+    ((2, 10, 10, 16), (1, 1, 16, 8), (2, 2), "VALID", -np.inf),   # 1x1: three of four classes skip the only tap
+    ((1, 7, 9, 4), (2, 2, 4, 3), (1, 3), "SAME", np.nan),
+])
+def test_strided_grad_input_with_non_finite_filter_weights(xs, ws, stride, padding, bad):
+    """The reference multiplies every tap with the dilated gradient, inserted zeros included
+    (cuda_kernel.cu:463-502): a weight that is inf or NaN turns 0 x w into NaN for every input
+    pixel, not only for the pixels whose residue class meets that tap.  The residue-class
+    sub-problems must reproduce that (NaNs compared as a class)."""
+    from approxtrain_amd import ApproxMulLut, functors
+    from tests.util import same_bits_or_both_nan
+    lut, L = ApproxMulLut.cached(lut_path("MBM", 7)), lut32("MBM", 7)
+    rng = np.random.default_rng(31)
+    w = rng.standard_normal(ws).astype(np.float32)
+    w[ws[0] - 1, 0, 1, 0] = bad          # one tap, one input channel
+    oh, _ = cpu.conv_geometry(xs[1], ws[0], stride[0], padding)
+    ow, _ = cpu.conv_geometry(xs[2], ws[1], stride[1], padding)
+    dy = rng.standard_normal((xs[0], oh, ow, ws[3])).astype(np.float32)
+    got = host(functors.convam_input_grad(lut, xs, dev(w), dev(dy), stride, padding))
+    want = cpu.conv2d_grad_input(L, 7, xs, w, dy, stride, padding)
+    assert np.all(same_bits_or_both_nan(got, want))
+    assert np.isnan(want[..., 1]).any() and np.isfinite(want[..., 0]).all()   # only that channel is hit
