@@ -76,6 +76,13 @@ def load_library():
     path = lib_path()
     if not os.path.exists(path):
         raise ImportError(f"{path} not built: run `make -C approxtrain_amd/csrc` (needs hipcc)")
+    # PyTorch ships its own copy of the HIP runtime.  Loading torch first makes libamsim.so bind to
+    # that copy, so the process holds one runtime and torch's device pointers and streams are valid
+    # in the library; loaded the other way round, the second runtime finds no device.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(path)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol

@@ -218,3 +218,23 @@ def test_strided_grad_input_with_non_finite_filter_weights(xs, ws, stride, paddi
     want = cpu.conv2d_grad_input(L, 7, xs, w, dy, stride, padding)
     assert np.all(same_bits_or_both_nan(got, want))
     assert np.isnan(want[..., 1]).any() and np.isfinite(want[..., 0]).all()   # only that channel is hit
+
+
+def test_library_loaded_before_torch_still_shares_its_runtime():
+    """A process that loads libamsim.so before it imports torch must not end up with two HIP
+    runtimes (torch bundles its own copy; the second one to start finds no device)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import approxtrain_amd\n"
+        "lib = approxtrain_amd.load_library()\n"            # before anything imports torch explicitly
+        "import torch\n"
+        "from approxtrain_amd import functors\n"
+        "a = torch.ones(8, 16, device='cuda'); b = torch.ones(16, 4, device='cuda')\n"
+        "out = functors.gemm('tests/golden/lut/ACC_7.bin', a, b)\n"
+        "print('sum', float(out.sum()))\n")
+    run = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert "sum 512.0" in run.stdout
