@@ -122,8 +122,8 @@ def torch_conv_reference(x, w, dy, strides, padding):
     Returns (y, dx, dw) as float64 numpy arrays. dy may be None."""
     import torch
     import torch.nn.functional as F
-    xt = torch.tensor(np.asarray(x, np.float64)).permute(0, 3, 1, 2).requires_grad_(True)
-    wt = torch.tensor(np.asarray(w, np.float64)).permute(3, 2, 0, 1).requires_grad_(True)
+    xt = torch.tensor(np.asarray(x, np.float64)).permute(0, 3, 1, 2).contiguous().requires_grad_(True)
+    wt = torch.tensor(np.asarray(w, np.float64)).permute(3, 2, 0, 1).contiguous().requires_grad_(True)
     if padding == "SAME":
         _, pt, pb = tf_same_pads(x.shape[1], w.shape[0], strides[0])
         _, pl, pr = tf_same_pads(x.shape[2], w.shape[1], strides[1])
