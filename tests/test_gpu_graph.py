@@ -76,3 +76,52 @@ def test_attention_and_dense_replay_from_a_graph():
         torch.cuda.synchronize()
         for got, want in zip(captured, eager):
             assert np.array_equal(_bits(got), _bits(want))
+
+
+def test_whole_training_step_with_autograd_and_optimizer_replays_from_a_graph():
+    """LeNet-5-shaped model through the layers: forward, loss, autograd backward and the SGD
+    update captured as one graph.  The loss of every replay must follow the eager run's
+    trajectory (same seeds, same data), step by step."""
+    from tests.test_gpu_training import _lenet
+    rng = np.random.default_rng(0)
+    protos = rng.standard_normal((10, 28, 28, 1)).astype(np.float32)
+    labels = rng.integers(0, 10, 128)
+    data = protos[labels] + 0.5 * rng.standard_normal((128, 28, 28, 1)).astype(np.float32)
+    x, y = torch.from_numpy(data).cuda(), torch.from_numpy(labels).cuda()
+
+    def trajectory(graphed, steps=12):
+        torch.manual_seed(0)
+        model = _lenet()
+        opt = torch.optim.SGD(model.parameters(), lr=0.05, momentum=0.9)
+
+        def step():
+            opt.zero_grad(set_to_none=False)
+            loss = torch.nn.functional.cross_entropy(model(x), y)
+            loss.backward()
+            opt.step()
+            return loss.detach()
+
+        losses = []
+        side = torch.cuda.Stream()                       # warm-up off the default stream, as capture requires
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                losses.append(float(step()))
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        if graphed:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_loss = step()
+            for _ in range(steps):
+                graph.replay()
+                torch.cuda.synchronize()
+                losses.append(float(static_loss))
+        else:
+            for _ in range(steps):
+                losses.append(float(step()))
+        return np.array(losses)
+
+    eager, replayed = trajectory(False), trajectory(True)
+    assert np.all(np.isfinite(eager)) and eager[-1] < eager[0]      # it trains
+    np.testing.assert_allclose(replayed, eager, rtol=2e-4, atol=1e-6)
