@@ -185,7 +185,7 @@ int amsim_convam_bias_act_f32(amsim_lut_t lut, const float *input_data, float *o
     d.p.B = batch; d.p.GH = out_rows; d.p.GW = out_cols;
     d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = in_depth;
     d.p.sy = stride_rows; d.p.sx = stride_cols; d.p.pt = filter_top_offset; d.p.pl = filter_left_offset;
-    d.p.dy = 1; d.p.dx = 1; d.p.VH = input_rows; d.p.VW = input_cols; d.p.SH = input_rows; d.p.SW = input_cols;
+    d.p.SH = input_rows; d.p.SW = input_cols;
     d.q.kind = Q_DENSE; d.q.base = filter; d.q.sk = out_depth; d.q.sj = 1;
     d.out = output_data; d.so_r = out_depth; d.so_j = 1;
     d.bias_j = bias; d.act = activation;
@@ -241,7 +241,7 @@ GemmDesc grad_input_phase(const GradInputGeometry &g, int py, int px, const floa
     d.p.B = g.batch; d.p.GH = y.n_out; d.p.GW = x.n_out;
     d.p.KH = y.taps; d.p.KW = x.taps; d.p.C = g.out_depth;
     d.p.sy = 1; d.p.sx = 1; d.p.pt = y.pad; d.p.pl = x.pad;
-    d.p.dy = 1; d.p.dx = 1; d.p.VH = g.out_rows; d.p.VW = g.out_cols; d.p.SH = g.out_rows; d.p.SW = g.out_cols;
+    d.p.SH = g.out_rows; d.p.SW = g.out_cols;
     d.q.kind = Q_FLIP; d.q.base = filter;
     d.q.KH = g.filter_rows; d.q.KW = g.filter_cols; d.q.IC = g.in_depth; d.q.OC = g.out_depth;
     d.q.TH = y.taps; d.q.TW = x.taps; d.q.fy0 = y.f0; d.q.fx0 = x.f0; d.q.fsy = g.stride_rows; d.q.fsx = g.stride_cols;
@@ -403,7 +403,7 @@ int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const floa
     d.p.B = batch; d.p.GH = out_rows; d.p.GW = out_cols;
     d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = in_depth;
     d.p.sy = stride_rows; d.p.sx = stride_cols; d.p.pt = filter_top_offset; d.p.pl = filter_left_offset;
-    d.p.SH = input_rows; d.p.SW = input_cols; d.p.VH = input_rows; d.p.VW = input_cols;
+    d.p.SH = input_rows; d.p.SW = input_cols;
     d.q.kind = Q_DENSE; d.q.base = grad; d.q.sk = out_depth; d.q.sj = 1;
     d.out = output; d.so_r = out_depth; d.so_j = 1;
     d.lane_first = true;  // P(input, grad)

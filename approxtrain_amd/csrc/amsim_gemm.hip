@@ -175,7 +175,7 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
 // ---------------------------------------------------------------------------
 // lane-operand row bookkeeping, kept in LDS: one int4 per local row.
 //   P_PATCH: {source offset of image b, y*sy - pt, x*sx - pl, source offset of the
-//            window origin (undilated sources)}; rows past the end get a y origin
+//            window origin}; rows past the end get a y origin
 //            far outside the source.
 //   P_GF:    {(fy*SW + fx)*C + c, fy, fx, 0}; rows past the end get fy far outside.
 // ---------------------------------------------------------------------------
@@ -354,9 +354,9 @@ void lutgemm_kernel(KArgs a)
         }
     };
 
-    // Undilated patch sources whose channel count is a multiple of the chunk depth: every
+    // Patch sources whose channel count is a multiple of the chunk depth: every
     // chunk lies inside one filter tap, so the tap offset and the window test are scalar work
-    const bool tap_uniform = PK == P_PATCH && STAGE == STAGE_K4 && a.p.dy == 1 && a.p.dx == 1 && (a.p.C % KC == 0);
+    const bool tap_uniform = PK == P_PATCH && STAGE == STAGE_K4 && (a.p.C % KC == 0);
 
     // Filter-gradient tiles that lie inside one (fy, fx) (channel count a multiple of the tile
     // height, tile fully inside R): wave-uniform window offset
@@ -396,16 +396,8 @@ void lutgemm_kernel(KArgs a)
                 } else {
                     const int4 ri = rowinfo[rl];
                     const int vy = ri.y + fy, vx = ri.z + fx;
-                    if (kvalid && (unsigned)vy < (unsigned)a.p.VH && (unsigned)vx < (unsigned)a.p.VW) {
-                        int sy_ = vy, sx_ = vx;
-                        bool on_grid = true;
-                        if (a.p.dy != 1 || a.p.dx != 1) {
-                            sy_ = vy / a.p.dy; sx_ = vx / a.p.dx;
-                            on_grid = (sy_ * a.p.dy == vy) && (sx_ * a.p.dx == vx);
-                        }
-                        if (on_grid)
-                            v = *reinterpret_cast<const uint4 *>(pbase + ri.x + (sy_ * a.p.SW + sx_) * a.p.C + c);
-                    }
+                    if (kvalid && (unsigned)vy < (unsigned)a.p.SH && (unsigned)vx < (unsigned)a.p.SW)
+                        v = *reinterpret_cast<const uint4 *>(pbase + ri.x + (vy * a.p.SW + vx) * a.p.C + c);
                 }
                 pv[4 * i + 0] = v.x; pv[4 * i + 1] = v.y; pv[4 * i + 2] = v.z; pv[4 * i + 3] = v.w;
                 sr.add(v.x); sr.add(v.y); sr.add(v.z); sr.add(v.w);
@@ -438,15 +430,8 @@ void lutgemm_kernel(KArgs a)
                 const int4 ri = rowinfo[rl];
                 const int vy = ri.y + fy, vx = ri.z + fx;
                 uint32_t v = 0;
-                if (kvalid && (unsigned)vy < (unsigned)a.p.VH && (unsigned)vx < (unsigned)a.p.VW) {
-                    int sy_ = vy, sx_ = vx;
-                    bool on_grid = true;
-                    if (a.p.dy != 1 || a.p.dx != 1) {
-                        sy_ = vy / a.p.dy; sx_ = vx / a.p.dx;
-                        on_grid = (sy_ * a.p.dy == vy) && (sx_ * a.p.dx == vx);
-                    }
-                    if (on_grid) v = f2u(pbase[ri.x + (sy_ * a.p.SW + sx_) * a.p.C + c]);
-                }
+                if (kvalid && (unsigned)vy < (unsigned)a.p.SH && (unsigned)vx < (unsigned)a.p.SW)
+                    v = f2u(pbase[ri.x + (vy * a.p.SW + vx) * a.p.C + c]);
                 pv[i] = v;
                 sr.add(v);
             }

@@ -64,13 +64,11 @@ struct PDesc {
     // P_DENSE: element (r, k) at base[r * sr + k * sk]
     int64_t sr = 0, sk = 0;
     // P_PATCH: r = (b, y, x) over [B, GH, GW], k = (fy, fx, c) over [KH, KW, C];
-    //          virtual source pixel (y*sy - pt + fy, x*sx - pl + fx) on a grid of
-    //          VH x VW that holds the real [B, SH, SW, C] source at multiples of
-    //          (dy, dx) and zeros elsewhere.
+    //          source pixel (y*sy - pt + fy, x*sx - pl + fx) of [B, SH, SW, C], zero outside.
     // P_GF:    r = (fy, fx, c) over [KH, KW, C], k = (b, y, x) over [B, GH, GW];
     //          source pixel (y*sy - pt + fy, x*sx - pl + fx) of [B, SH, SW, C].
     int B = 0, GH = 0, GW = 0, KH = 0, KW = 0, C = 0;
-    int sy = 1, sx = 1, pt = 0, pl = 0, dy = 1, dx = 1, VH = 0, VW = 0, SH = 0, SW = 0;
+    int sy = 1, sx = 1, pt = 0, pl = 0, SH = 0, SW = 0;
 };
 
 struct QDesc {
