@@ -370,9 +370,8 @@ void lutgemm_kernel(KArgs a)
     }
 
     uint32_t pv[ELEMS];
-    auto load_chunk = [&](int ch) -> int {
+    auto load_chunk = [&](int ch) {
         const int64_t k0 = (int64_t)ch * KC;
-        SafeRange sr;
         if (STAGE == STAGE_K4) {
             // thread -> (row, quad of 4 consecutive k); all four share (fy, fx) because C % 4 == 0
             const int kq = (tid & (KC / 4 - 1)) * 4;
@@ -400,7 +399,6 @@ void lutgemm_kernel(KArgs a)
                         v = *reinterpret_cast<const uint4 *>(pbase + ri.x + (vy * a.p.SW + vx) * a.p.C + c);
                 }
                 pv[4 * i + 0] = v.x; pv[4 * i + 1] = v.y; pv[4 * i + 2] = v.z; pv[4 * i + 3] = v.w;
-                sr.add(v.x); sr.add(v.y); sr.add(v.z); sr.add(v.w);
             }
             if (PK == P_DENSE) dptr += dchunk;
         } else if (PK == P_DENSE) {
@@ -415,7 +413,6 @@ void lutgemm_kernel(KArgs a)
                     if (k0 + kk < a.K && drow < dvalid_rows) v = f2u(dptr[(int64_t)i * dstep]);
                 }
                 pv[i] = v;
-                sr.add(v);
             }
             dptr += dchunk;
         } else if (PK == P_PATCH) {  // STAGE_K: this thread's k is fixed for the chunk
@@ -433,7 +430,6 @@ void lutgemm_kernel(KArgs a)
                 if (kvalid && (unsigned)vy < (unsigned)a.p.SH && (unsigned)vx < (unsigned)a.p.SW)
                     v = f2u(pbase[ri.x + (vy * a.p.SW + vx) * a.p.C + c]);
                 pv[i] = v;
-                sr.add(v);
             }
         } else {  // P_GF, staged along r: this thread stages ELEMS consecutive k (pixels) of its row
             const int rl = tid & (ROWS - 1);
@@ -466,7 +462,6 @@ void lutgemm_kernel(KArgs a)
                         uint32_t v = 0;
                         if (i < kleft && row_ok && (unsigned)ix < (unsigned)a.p.SW) v = f2u((pbase + soff)[chan]);
                         pv[i] = v;
-                        sr.add(v);
                         ix += a.p.sx;
                         soff += step;
                     }
@@ -477,7 +472,6 @@ void lutgemm_kernel(KArgs a)
                     if (i < kleft && (unsigned)iy < (unsigned)a.p.SH && (unsigned)ix < (unsigned)a.p.SW)
                         v = f2u((pbase + soff)[chan]);
                     pv[i] = v;
-                    sr.add(v);
                     if (++x == a.p.GW) {
                         x = 0;
                         if (++y == a.p.GH) { y = 0; ++b; }
@@ -500,13 +494,20 @@ void lutgemm_kernel(KArgs a)
                             v = f2u(pbase[((b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C + ri.x]);
                     }
                     pv[i] = v;
-                    sr.add(v);
                     if (++x == a.p.GW) { x = 0; if (++y == a.p.GH) { y = 0; ++b; } }
                 }
             }
         }
         if (PK == P_PATCH) advance_chunk_base();
-        return sr.unsafe() ? 1 : 0;
+    };
+    // Does the chunk held in pv[] contain an operand the fast product path cannot take?  Evaluated
+    // when the tile is stored, not when it is loaded: the loads stay in flight during the MACs of
+    // the chunk before instead of being waited for straight away.
+    auto staged_unsafe = [&]() -> bool {
+        SafeRange sr;
+#pragma unroll
+        for (int i = 0; i < ELEMS; ++i) sr.add(pv[i]);
+        return sr.unsafe();
     };
     auto store_chunk = [&]() {
         if (STAGE == STAGE_K4) {
@@ -538,8 +539,7 @@ void lutgemm_kernel(KArgs a)
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[j] = 0.0f;
 
-    int unsafe = 0;
-    if (ch_begin < ch_end) unsafe = load_chunk(ch_begin);
+    if (ch_begin < ch_end) load_chunk(ch_begin);
     // the LUT copies started above have landed in LDS once the vector-memory counter drains;
     // the barriers at the top of the first trip then order them against every wave's gathers
     if (!LUTG) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -563,11 +563,11 @@ void lutgemm_kernel(KArgs a)
         // Unsafe operands are rare: whoever staged one raises the chunk's flag (slot = chunk
         // parity); the slot of the previous chunk is cleared for the chunk after this one,
         // ordered against its writers by the barrier at the top of the next trip.
-        if (unsafe) pflag[ch & 1] = 1u;
+        if (staged_unsafe()) pflag[ch & 1] = 1u;
         __syncthreads();
         const uint32_t p_unsafe = __builtin_amdgcn_readfirstlane(pflag[ch & 1]);
         if (tid == 0) pflag[(ch & 1) ^ 1] = 0u;
-        if (ch + 1 < ch_end) unsafe = load_chunk(ch + 1);  // in flight during the MACs below
+        if (ch + 1 < ch_end) load_chunk(ch + 1);  // in flight during the MACs below
         if (!active) continue;
         const uint32_t q_unsafe = qflags[ch];
         const size_t qoff = (size_t)ch * KC * QT;
