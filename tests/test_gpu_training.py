@@ -57,3 +57,52 @@ def test_lenet_learns_a_synthetic_problem():
     assert acc > 0.8, acc
     # every parameter received a gradient through the approximate ops
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+
+
+def test_resnet_bottleneck_block_runs_through_the_library():
+    """A ResNet-50 bottleneck (1x1 reduce -> 3x3 -> 1x1 expand, identity shortcut, stride-2 variant
+    with a projection shortcut): every convolution, forward and backward, is an AMConv2D.  Each
+    layer's output is checked against the oracle on that layer's actual input, and the block's
+    parameters all receive finite gradients."""
+    import approxtrain_amd
+    from approxtrain_amd.layers import AMConv2D
+    from oracle import cpu
+    from tests.gpu_util import host, lut32
+    lib = approxtrain_amd.load_library()
+    L = lut32("MBM", 7)
+
+    class Bottleneck(torch.nn.Module):
+        def __init__(self, cin, mid, cout, stride):
+            super().__init__()
+            conv = lambda f, k, s, a, c: AMConv2D(f, k, strides=s, padding="same", activation=a, mant_mul_lut=MBM, in_channels=c)
+            self.a = conv(mid, 1, 1, "relu", cin)
+            self.b = conv(mid, 3, stride, "relu", mid)
+            self.c = conv(cout, 1, 1, None, mid)
+            self.proj = conv(cout, 1, stride, None, cin) if (stride != 1 or cin != cout) else None
+
+        def forward(self, x):
+            self.seen = [x]
+            h = self.a(x); self.seen.append(h)
+            h = self.b(h); self.seen.append(h)
+            h = self.c(h); self.seen.append(h)
+            short = x if self.proj is None else self.proj(x)
+            return torch.relu(h + short)
+
+    torch.manual_seed(1)
+    lib.amsim_set_split_k(0)
+    try:
+        for cin, mid, cout, stride, hw in ((64, 16, 64, 1, 14), (64, 32, 128, 2, 14)):
+            block = Bottleneck(cin, mid, cout, stride).cuda()
+            x = torch.randn(2, hw, hw, cin, device="cuda", requires_grad=True)
+            y = block(x)
+            assert tuple(y.shape) == (2, hw // stride, hw // stride, cout)
+            for layer, xin, out in zip((block.a, block.b, block.c), block.seen[:-1], block.seen[1:]):
+                want = cpu.conv2d_fwd(L, 7, host(xin), host(layer.kernel), tuple(layer.strides), "SAME") + host(layer.bias)
+                if layer.activation is not None:
+                    want = np.where(want < 0, np.float32(0), want)
+                assert np.array_equal(host(out).view(np.uint32), want.astype(np.float32).view(np.uint32))
+            y.square().mean().backward()
+            assert torch.isfinite(x.grad).all() and float(x.grad.abs().sum()) > 0
+            assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in block.parameters())
+    finally:
+        lib.amsim_set_split_k(1)
