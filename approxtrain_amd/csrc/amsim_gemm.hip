@@ -900,7 +900,8 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
     pl.Rp = (R + rows - 1) / rows * rows;
     const int64_t rowtiles = pl.Rp / rows;
     const int64_t G = ((jchunks + wc - 1) / wc) * batch;
-    const int64_t slots = DEVICE_CUS * (pl.WR == 1 ? waves64 : 2);  // resident workgroups (the 256-row kernels run 2 per CU)
+    // resident workgroups: the 256-row kernels hold 53 KB of LDS and up to 170 VGPRs, three fit a CU
+    const int64_t slots = DEVICE_CUS * (pl.WR == 1 ? waves64 : 3);
 
     Shape sh;
     sh.cps = pl.nchunks;
@@ -910,7 +911,7 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
         // one chunk of one workgroup on a full machine, and one pass over the output, in seconds
         const double chunk_s = (double)rows * (wc * pl.TN) * KC * slots / 13.0e12;
         const double pass_s = 2.0 * (double)pl.Rp * pl.Jp * batch * sizeof(float) / 3.0e12;
-        sh = shape_work(rowtiles, G, pl.nchunks, slots, pl.WR == 1, pass_s / chunk_s);
+        sh = shape_work(rowtiles, G, pl.nchunks, slots, true, pass_s / chunk_s);
     }
     pl.nsplit = sh.nsplit;
     pl.chunks_per_split = sh.cps;
