@@ -254,6 +254,8 @@ def _plan(M, N, K, batch=1, ta=0, tb=0):
     (512, 512, 8192, "split"),          # few outputs, long reduction
     (51200, 64, 128, "whole"),          # short reduction: nothing to gain from splitting
     (40, 6, 50000, "split"),            # one row tile
+    (200704, 1, 150, "tail"),           # 256-row workgroups (one narrow column group): 768 slots + a split tail
+    (50176, 6, 400, "split"),           # 256-row workgroups, reduction split three ways
 ])
 def test_planner_paths_match_the_oracle(amd, M, N, K, expect):
     """The work-shaping decisions (reduction split, tail rows split further, both with partial sums)
@@ -270,7 +272,7 @@ def test_planner_paths_match_the_oracle(amd, M, N, K, expect):
     B = rng.standard_normal((K, N)).astype(np.float32)
     lut = ApproxMulLut.cached(lut_path("MBM", 7))
     got = host(amd.gemm(lut, dev(A), dev(B)))
-    rows = np.unique(np.concatenate([np.arange(min(M, 70)), rng.integers(0, M, 60), np.arange(max(M - 130, 0), M)]))
+    rows = np.unique(np.concatenate([np.arange(min(M, 70)), rng.integers(0, M, 60), np.arange(max(M - 300, 0), M)]))
     L = lut32("MBM", 7)
     want = cpu.gemm(L, 7, A[rows].copy(), B)
     assert_close_sum_abs(got[rows], want, cpu.gemm_abs(L, 7, A[rows].copy(), B), 1e-5)
