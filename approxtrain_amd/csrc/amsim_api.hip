@@ -544,6 +544,7 @@ int amsim_attention_f32(amsim_lut_t lut, const float *q, const float *k, const f
                         size_t workspace_bytes, void *stream)
 {
     const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
     if (!attn_shape_ok(s)) return fail(AMSIM_ERR_INVALID, "negative extent");
     if (!(divisor > 0.0f)) return fail(AMSIM_ERR_INVALID, "the score divisor must be positive");
     if (mask && (mask_batch_div < 1 || mask_batch_stride < 0 || mask_row_stride < 0))
@@ -575,6 +576,7 @@ int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, co
                              void *stream)
 {
     const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
     if (!attn_shape_ok(s)) return fail(AMSIM_ERR_INVALID, "negative extent");
     if (!(divisor > 0.0f)) return fail(AMSIM_ERR_INVALID, "the score divisor must be positive");
     if (batch == 0) return AMSIM_OK;

@@ -86,6 +86,37 @@ def test_attention_mask_layout_rejects_shapes_that_do_not_broadcast():
         _mask_layout(torch.zeros(2, 3, 5, 7, 1), (2, 3), 5, 7, torch.device("cpu"))
 
 
+def test_no_entry_point_crashes_on_null_or_odd_arguments():
+    """Every compute entry point called with a null LUT handle, null tensors and extents of
+    0 / 1 / -1 / 7 must come back with a status (no launch, no crash), and every workspace query
+    with a size (0 for impossible extents)."""
+    lib = approxtrain_amd.load_library()
+    other = {"amsim_status_string", "amsim_last_error", "amsim_device_info", "amsim_lut_load_file", "amsim_lut_create",
+             "amsim_lut_destroy", "amsim_lut_mant_width", "amsim_lut_params", "amsim_lut_generate",
+             "amsim_lut_generate_builtin", "amsim_microbench", "amsim_calibration_copy", "amsim_set_split_k",
+             "amsim_conv_geometry", "amsim_gemm_plan_info"}
+    for name, (res, args) in _lib.SIGNATURES.items():
+        if name in other:
+            continue
+        for fill in (0, 1, -1, 7):
+            vals = []
+            for a in args:
+                if a is C.c_size_t:
+                    vals.append(max(fill, 0))
+                elif a in (C.c_int, C.c_int64):
+                    vals.append(fill)
+                elif a is C.c_float:
+                    vals.append(1.0)
+                else:
+                    vals.append(None)
+            out = getattr(lib, name)(*vals)
+            if name.endswith("_workspace_bytes"):
+                assert out >= 0 and (fill > 0 or out == 0), (name, fill, out)
+            else:
+                assert out == 1, (name, fill, out)                      # AMSIM_ERR_INVALID: nothing was launched
+                assert lib.amsim_last_error(), name
+
+
 def test_tensorflow_bridge_uses_only_declared_entry_points():
     """The TensorFlow bridge cannot be compiled here (no TensorFlow); at least every C-ABI
     call in it must name an entry point the header declares, and every GPU functor of the
