@@ -33,6 +33,7 @@ SIGNATURES = {
     "amsim_lut_destroy": (_i, [_p]),
     "amsim_lut_mant_width": (_i, [_p]),
     "amsim_lut_params": (_i, [_p, C.POINTER(C.c_uint32), C.POINTER(_i), C.POINTER(_i)]),
+    "amsim_lut_set_split_k": (_i, [_p, _i]),
     "amsim_lut_generate": (_i, [_p, _p, _i, _i, _p, _sz]),
     "amsim_lut_generate_builtin": (_i, [C.c_char_p, _i, _i, _p, _sz]),
     "amsim_mul_f32": (_i, [_p, _f, _f, _f, _sz, _p]),
@@ -62,6 +63,7 @@ SIGNATURES = {
     "amsim_conv_geometry": (_i, [_i, _i, _i, _i, C.POINTER(_i), C.POINTER(_i)]),
     "amsim_set_split_k": (_i, [_i]),
     "amsim_calibration_copy": (_i, [_f, _f, _sz, _p]),
+    "amsim_microbench_wide": (_i, [_i, _i, _i, _i, _p, _p, _sz, _f, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "amsim_microbench": (_i, [_i, _i, _i, _i, _p, _f, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
 }
 

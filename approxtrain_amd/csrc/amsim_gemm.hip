@@ -47,7 +47,8 @@ constexpr int WG_THREADS = 256;
 constexpr int LUT_LDS_BYTES = 16384 + 128;   // 2^(2m) entries + one all-zero row of 2^m entries (m <= 7)
 constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels are compiled for
 constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
-constexpr int DEVICE_CUS = 256;               // MI355X; only steers work splitting, never correctness
+constexpr double MACS_PER_CU_S = 13.0e12 / 256;  // planner's price of a MAC: what one compute unit sustains
+constexpr double PARTIAL_BYTES_PER_S = 3.0e12;   // planner's price of writing + re-reading partial sums
 
 static std::atomic<int> g_split_k{1};
 
@@ -91,7 +92,10 @@ struct KArgs {
     int m;
     int lane_first;
     const uint32_t *qw;      // [qb][Jp/16][Kp][16]  sign|exponent | row offset
-    const uint32_t *qraw;    // same layout, raw bits
+    const QDesc *qdesc;      // the uniform operand where it lies (a copy of its descriptor in device memory, written
+                             // by the pre-pass): flagged chunks read its raw bits from there.  Kept behind a pointer
+                             // so that its fields are loaded inside the rare path only and cost the inner loop no
+                             // scalar registers.
     const uint32_t *qflags;  // [qb][Jp/16][nchunks]
     int q_batches;
     int64_t R, J, K;
@@ -120,25 +124,39 @@ struct QArgs {
     int64_t K, J;
     int Jp, nchunks, m;
     uint32_t *qw;
-    uint32_t *qraw;
     uint32_t *qflags;
+    QDesc *qdesc_out;
 };
+
+// raw bits of uniform-operand element (k, j) of batch item `base`; zero outside K x J
+// (k < 2^31 and j < 2^24 on every path that gets here)
+template <typename QD>
+__device__ __forceinline__ uint32_t q_raw_bits(const QD &q, const float *base, uint32_t K, uint32_t J, uint32_t k, uint32_t j)
+{
+    if (k >= K || j >= J) return 0u;
+    if (q.kind == Q_DENSE) return f2u(base[(int64_t)k * q.sk + (int64_t)j * q.sj]);
+    const uint32_t oc = k % (uint32_t)q.OC, t = k / (uint32_t)q.OC;
+    const int fx = q.fx0 + (int)(t % (uint32_t)q.TW) * q.fsx, fy = q.fy0 + (int)(t / (uint32_t)q.TW) * q.fsy;
+    return f2u(base[(((int64_t)(q.KH - 1 - fy) * q.KW + (q.KW - 1 - fx)) * q.IC + j) * q.OC + oc]);
+}
 
 // One wavefront per (32-row chunk, 16-column tile): decodes the tile, writes it
 // in the tile-major layout the main kernel streams, and flags the tile-chunk
-// if it holds an operand the fast product path cannot take.
+// if it holds an operand the fast product path cannot take.  blockIdx.x runs over
+// (chunk, group of four column tiles), blockIdx.y over the batch.
 __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
 {
-    const int ch = blockIdx.x, qb = blockIdx.z;
-    const int lane = threadIdx.x & 63;
-    const int jt = blockIdx.y * (WG_THREADS / 64) + (threadIdx.x >> 6);
     const int ntiles = a.Jp / QT;
+    const int tgroups = (ntiles + WG_THREADS / 64 - 1) / (WG_THREADS / 64);
+    const int ch = blockIdx.x / tgroups, qb = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int jt = (blockIdx.x % tgroups) * (WG_THREADS / 64) + (threadIdx.x >> 6);
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *a.qdesc_out = a.q;
     if (jt >= ntiles) return;
     const float *base = a.q.base + (int64_t)qb * a.q.batch_stride;
     const size_t Kp = (size_t)a.nchunks * KC;
     const size_t tile = ((size_t)qb * ntiles + jt) * Kp * QT + (size_t)ch * KC * QT;
     uint32_t *qw = a.qw + tile;
-    uint32_t *qraw = a.qraw + tile;
     // lanes follow the source's contiguous direction
     const bool k_fast = (a.q.kind == Q_DENSE && a.q.sk == 1 && a.q.sj != 1) || (a.q.kind == Q_FLIP);
     int unsafe = 0;
@@ -148,25 +166,12 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
         int kk, jj;
         if (k_fast) { kk = e % KC; jj = e / KC; }
         else { jj = e % QT; kk = e / QT; }
-        const int64_t k = (int64_t)ch * KC + kk;
-        const int64_t j = (int64_t)jt * QT + jj;
-        uint32_t raw = 0;
-        if (k < a.K && j < a.J) {
-            if (a.q.kind == Q_DENSE) {
-                raw = f2u(base[k * a.q.sk + j * a.q.sj]);
-            } else {
-                const int oc = (int)(k % a.q.OC);
-                const int t = (int)(k / a.q.OC);
-                const int fx = a.q.fx0 + (t % a.q.TW) * a.q.fsx, fy = a.q.fy0 + (t / a.q.TW) * a.q.fsy;
-                raw = f2u(base[(((int64_t)(a.q.KH - 1 - fy) * a.q.KW + (a.q.KW - 1 - fx)) * a.q.IC + j) * a.q.OC + oc]);
-            }
-        }
+        const uint32_t raw = q_raw_bits(a.q, base, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)ch * KC + kk, (uint32_t)jt * QT + jj);
         unsafe |= operand_unsafe(raw) ? 1 : 0;
         // zero (and padding) elements select the all-zero LUT row that follows the table:
         // their product term is then exactly +-0 without a test in the inner loop
         const uint32_t mant = (raw & 0x7fffffffu) ? ((raw & 0x7fffffu) >> (23 - a.m)) : (1u << a.m);
         qw[kk * QT + jj] = (raw & 0xff800000u) | (mant << a.m);
-        qraw[kk * QT + jj] = raw;  // the exact path of a chunk flagged by EITHER operand reads these
     }
     const int any = __any(unsafe);
     if (lane == 0) a.qflags[((size_t)qb * ntiles + jt) * a.nchunks + ch] = (uint32_t)any;
@@ -289,7 +294,6 @@ void lutgemm_kernel(KArgs a)
     // wave-uniform reads become scalar loads (s_load) into SGPRs.
     const size_t qtile = ((size_t)qb * (a.Jp / QT) + (size_t)(j0 / QT)) * Kp * QT + (size_t)(j0 % QT);
     const cq1_t qw = (cq1_t)(uintptr_t)(a.qw + qtile);
-    const cq1_t qraw = (cq1_t)(uintptr_t)(a.qraw + qtile);
     const cq1_t qflags = (cq1_t)(uintptr_t)(a.qflags + ((size_t)qb * (a.Jp / QT) + (size_t)(j0 / QT)) * a.nchunks);
 
     const int ch_begin = split * seg_cps;
@@ -619,19 +623,25 @@ void lutgemm_kernel(KArgs a)
                 qrow += KG * QT;
             }
         } else {
-            cq1_t qrow = qraw + qoff;
+            // rare: the uniform operand's raw bits come from where it lies, not from the workspace
             const uint32_t *Pt = reinterpret_cast<const uint32_t *>(Pt4);
+            // (the descriptor was written by an earlier kernel: read it through the scalar cache)
+            const __attribute__((address_space(4))) QDesc &qd = *(const __attribute__((address_space(4))) QDesc *)(uintptr_t)a.qdesc;
+            const float *qsrc = qd.base + (int64_t)qb * qd.batch_stride;
+#pragma unroll 1
             for (int kk = 0; kk < KC; ++kk) {
                 const uint32_t raw = Pt[((kk >> 2) * GS + lrow) * 4 + (kk & 3)];
                 const uint32_t ia = (raw & 0x7fffffu) >> mshift;
+#pragma unroll 1
+                for (int jb = 0; jb < TN; jb += 4) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const uint32_t qr = qrow[j];
-                    const uint32_t li = (((qr & 0x7fffffu) >> mshift) << m) + ia;
-                    const uint32_t e16 = (LUTG ? (uint32_t)lut_g[li] : (uint32_t)lut_s[li]) << ESHIFT;
-                    acc[j] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
+                    for (int j = jb; j < jb + 4 && j < TN; ++j) {
+                        const uint32_t qr = q_raw_bits(qd, qsrc, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)ch * KC + kk, (uint32_t)(j0 + j));
+                        const uint32_t li = (((qr & 0x7fffffu) >> mshift) << m) + ia;
+                        const uint32_t e16 = (LUTG ? (uint32_t)lut_g[li] : (uint32_t)lut_s[li]) << ESHIFT;
+                        acc[j] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
+                    }
                 }
-                qrow += QT;
             }
         }
     }
@@ -796,7 +806,7 @@ struct Plan {
     int64_t Rp;                    // padded rows
     int64_t rows_main;             // rows covered by the main part (== R when there is no tail)
     int tail_nsplit, tail_chunks_per_split;
-    size_t off_qw, off_qraw, off_flags, off_partial_main, off_partial_tail, total;
+    size_t off_qw, off_flags, off_qdesc, off_partial_main, off_partial_tail, total;
 };
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -862,7 +872,7 @@ static Shape shape_work(int64_t rowtiles, int64_t G, int n, int64_t slots, bool 
     return best;
 }
 
-static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64);
+static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int cus);
 
 // Plans are pure functions of their arguments; the last few are remembered per thread so that
 // the workspace query and the call that follows it do not repeat the search.
@@ -873,19 +883,20 @@ static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches,
     struct Slot { Key k; Plan p; bool used = false; };
     static thread_local Slot memo[8];
     static thread_local unsigned next = 0;
-    const Key key{R, J, K, batch, q_batches, (split_k ? 1 : 0) | (waves64 << 1)};
+    const int cus = device_compute_units();
+    const Key key{R, J, K, batch, q_batches, (split_k ? 1 : 0) | (waves64 << 1) | (cus << 8)};
     for (const Slot &sl : memo)
         if (sl.used && sl.k.R == R && sl.k.J == J && sl.k.K == K && sl.k.batch == batch && sl.k.qb == q_batches &&
             sl.k.split == key.split)
             return sl.p;
     Slot &sl = memo[next++ % 8];
     sl.k = key;
-    sl.p = compute_plan(R, J, K, batch, q_batches, split_k, waves64);
+    sl.p = compute_plan(R, J, K, batch, q_batches, split_k, waves64, cus);
     sl.used = true;
     return sl.p;
 }
 
-static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64)
+static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int cus)
 {
     Plan pl{};
     // Narrow outputs (one column group) stack four row tiles per workgroup and shrink the
@@ -901,7 +912,7 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
     const int64_t rowtiles = pl.Rp / rows;
     const int64_t G = ((jchunks + wc - 1) / wc) * batch;
     // resident workgroups: the 256-row kernels hold 53 KB of LDS and up to 170 VGPRs, three fit a CU
-    const int64_t slots = DEVICE_CUS * (pl.WR == 1 ? waves64 : 3);
+    const int64_t slots = (int64_t)cus * (pl.WR == 1 ? waves64 : 3);
 
     Shape sh;
     sh.cps = pl.nchunks;
@@ -909,8 +920,8 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
     sh.tail_cps = pl.nchunks;
     if (split_k && pl.nchunks > 1) {
         // one chunk of one workgroup on a full machine, and one pass over the output, in seconds
-        const double chunk_s = (double)rows * (wc * pl.TN) * KC * slots / 13.0e12;
-        const double pass_s = 2.0 * (double)pl.Rp * pl.Jp * batch * sizeof(float) / 3.0e12;
+        const double chunk_s = (double)rows * (wc * pl.TN) * KC * slots / (MACS_PER_CU_S * cus);
+        const double pass_s = 2.0 * (double)pl.Rp * pl.Jp * batch * sizeof(float) / PARTIAL_BYTES_PER_S;
         sh = shape_work(rowtiles, G, pl.nchunks, slots, true, pass_s / chunk_s);
     }
     pl.nsplit = sh.nsplit;
@@ -922,8 +933,8 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
     const size_t plane = (size_t)pl.nchunks * KC * pl.Jp;
     size_t off = 0;
     pl.off_qw = off;      off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
-    pl.off_qraw = off;    off = align256(off + (size_t)q_batches * plane * sizeof(uint32_t));
     pl.off_flags = off;   off = align256(off + (size_t)q_batches * (pl.Jp / QT) * std::max(pl.nchunks, 1) * sizeof(uint32_t));
+    pl.off_qdesc = off;   off = align256(off + sizeof(QDesc));
     const int64_t main_rows_p = sh.main_rowtiles * rows, tail_rows_p = pl.Rp - main_rows_p;
     pl.off_partial_main = off;
     if (pl.nsplit > 1) off = align256(off + (size_t)pl.nsplit * batch * main_rows_p * pl.Jp * sizeof(float));
@@ -1012,6 +1023,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     if (d.R == 0 || d.J == 0 || d.batch == 0) return AMSIM_OK;
     if ((lut.m <= 7 && lut.img_ab == nullptr) || (lut.m > 7 && lut.img16_ab == nullptr))
         return fail(AMSIM_ERR_UNSUPPORTED, "LUT handle holds no device image for the GEMM path");
+    if (const int rc = check_lut_device(lut)) return rc;
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
         RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0,
@@ -1024,8 +1036,9 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     }
     if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
-    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, g_split_k.load() != 0 && !d.no_split,
-                              waves64_of(d.p, d.K));
+    // the handle's own setting wins over the process default (read once per call)
+    const bool may_split = (lut.split_k >= 0 ? lut.split_k != 0 : g_split_k.load() != 0) && !d.no_split;
+    const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, may_split, waves64_of(d.p, d.K));
     // the size the query returns (valid for either split mode), not just this plan's
     const size_t need = d.no_split ? pl.total : gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
     if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need)
@@ -1037,10 +1050,12 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     qa.q = d.q;
     qa.K = d.K; qa.J = d.J; qa.Jp = pl.Jp; qa.nchunks = pl.nchunks; qa.m = lut.m;
     qa.qw = reinterpret_cast<uint32_t *>(ws + pl.off_qw);
-    qa.qraw = reinterpret_cast<uint32_t *>(ws + pl.off_qraw);
     qa.qflags = reinterpret_cast<uint32_t *>(ws + pl.off_flags);
+    qa.qdesc_out = reinterpret_cast<QDesc *>(ws + pl.off_qdesc);
     if (d.q.batches > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
-    q_prepass_kernel<<<dim3(pl.nchunks, (pl.Jp / QT + 3) / 4, d.q.batches), WG_THREADS, 0, stream>>>(qa);
+    const int64_t prepass_wgs = (int64_t)pl.nchunks * ((pl.Jp / QT + 3) / 4);
+    if (prepass_wgs >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "uniform operand exceeds the grid limit");
+    q_prepass_kernel<<<dim3((unsigned)prepass_wgs, (unsigned)d.q.batches), WG_THREADS, 0, stream>>>(qa);
     AMSIM_HIP_CHECK(hipGetLastError());
 
     KArgs ka{};
@@ -1050,7 +1065,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.lut_bytes = (int)(((size_t)1 << (2 * lut.m)) + ((size_t)1 << lut.m) + 15) / 16 * 16;
     ka.m = lut.m;
     ka.lane_first = d.lane_first ? 1 : 0;
-    ka.qw = qa.qw; ka.qraw = qa.qraw; ka.qflags = qa.qflags;
+    ka.qw = qa.qw; ka.qdesc = qa.qdesc_out; ka.qflags = qa.qflags;
     ka.q_batches = d.q.batches;
     ka.R = d.R; ka.J = d.J; ka.K = d.K;
     ka.Jp = pl.Jp; ka.nchunks = pl.nchunks;
@@ -1120,6 +1135,7 @@ __global__ __launch_bounds__(WG_THREADS) void mul_kernel(const uint32_t *lut32, 
 int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream)
 {
     if (n == 0) return AMSIM_OK;
+    if (const int rc = check_lut_device(lut)) return rc;
     const unsigned blocks = (unsigned)std::min<size_t>((n + WG_THREADS - 1) / WG_THREADS, 65535u * 16u);
     mul_kernel<<<blocks, WG_THREADS, 0, stream>>>(lut.lut32, lut.m, a, b, out, n);
     AMSIM_HIP_CHECK(hipGetLastError());

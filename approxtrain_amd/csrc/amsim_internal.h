@@ -32,6 +32,7 @@ int fail(int status, const std::string &msg);
 struct Lut {
     int m = 0;
     int device = 0;
+    int split_k = -1;  // how reductions may be run for calls through this handle: -1 process default, 0 whole, 1 split
     size_t entries = 0;
     uint8_t *img_ab = nullptr;
     uint8_t *img_ba = nullptr;
@@ -107,6 +108,12 @@ struct GemmDesc {
     OutMap omap;
     bool no_split = false;  // keep every reduction whole (needs no partial-sum workspace)
 };
+
+// Compute units of the current device (read once per device; 256 when no device answers, which
+// only steers work splitting, never correctness).
+int device_compute_units();
+// AMSIM_OK when the handle's images live on the current device, else AMSIM_ERR_INVALID.
+int check_lut_device(const Lut &lut);
 
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
 void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int64_t info[8]);

@@ -3,6 +3,7 @@
 // texture object of cuda/approx_mul_lut.cu:24-48).
 #include "amsim_internal.h"
 
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <fstream>
@@ -21,6 +22,35 @@ int fail(int status, const std::string &msg)
 }
 
 const std::string &last_error() { return g_last_error; }
+
+int device_compute_units()
+{
+    constexpr int MAX_DEV = 64;
+    static std::atomic<int> cus[MAX_DEV];  // 0 = not read yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    cus[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
+int check_lut_device(const Lut &lut)
+{
+    int dev = 0;
+    AMSIM_HIP_CHECK(hipGetDevice(&dev));
+    if (dev != lut.device)
+        return fail(AMSIM_ERR_INVALID, "LUT handle was created on device " + std::to_string(lut.device) +
+                                           ", the current device is " + std::to_string(dev));
+    return AMSIM_OK;
+}
 
 // entries: one (carry, mantissa) pair per (ma, mb), mantissa in m bits
 void lut_free(Lut &l);
@@ -211,6 +241,14 @@ int amsim_lut_destroy(amsim_lut_t lut)
 }
 
 int amsim_lut_mant_width(amsim_lut_t lut) { return lut ? lut->l.m : -1; }
+
+int amsim_lut_set_split_k(amsim_lut_t lut, int mode)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (mode < -1 || mode > 1) return fail(AMSIM_ERR_INVALID, "split mode must be -1 (process default), 0 or 1");
+    lut->l.split_k = mode;
+    return AMSIM_OK;
+}
 
 int amsim_lut_params(amsim_lut_t lut, uint32_t *mant_mask, int *a_shift, int *b_shift)
 {

@@ -75,6 +75,15 @@ int amsim_lut_destroy(amsim_lut_t lut);
 int amsim_lut_mant_width(amsim_lut_t lut);
 /* the derived fields of approx_mul_lut.h:26-28 */
 int amsim_lut_params(amsim_lut_t lut, uint32_t *mant_mask, int *a_shift, int *b_shift);
+/* How calls through this handle may run their reductions (no counterpart in the reference):
+ * 0 = every output is one sequential FP32 chain in ascending reduction index, bit-identical to
+ * a sequential CPU loop; 1 = problems with few outputs, and the tail rows of large ones, may
+ * split the reduction across workgroups (partial sums added in a fixed order: reproducible run
+ * to run, within 1e-5 * sum|products| of the sequential chain); -1 (initial value) = follow the
+ * process default of amsim_set_split_k.  The mode is read once per call; a workspace sized by
+ * the *_workspace_bytes queries is large enough for either mode.  Use one handle per thread
+ * (handles are cheap) when threads need different modes. */
+int amsim_lut_set_split_k(amsim_lut_t lut, int mode);
 
 /* ---- LUT generation (host side): replaces lut/lut_gen.cc:86-127 + lut/lut_gen.sh
  * A table holds, for every pair (i, j) of m-bit mantissas, the product of 1.i and
@@ -225,9 +234,8 @@ int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, co
 int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, int *out_size, int *pad_before);
 
 /* ---- knobs and measurement helpers (no counterpart in the reference) ----------
- * amsim_set_split_k(0) forces every reduction to stay one sequential chain per
- * output (bit-identical to a sequential CPU loop); 1 (default) lets problems
- * with few outputs split the reduction across workgroups. */
+ * amsim_set_split_k sets the process default that handles in mode -1 follow (see
+ * amsim_lut_set_split_k for the two modes and their tolerance); the initial default is 1. */
 int amsim_set_split_k(int mode);
 /* How a GEMM of this shape would be run when reductions may be split (contiguous, aligned
  * operands assumed): info = {outputs per lane, row tiles per workgroup, splits of the main part's
@@ -238,11 +246,23 @@ int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K
  * (kind 0 / 10: independent FP32 FMAs; 11..13: v_add_u32, v_lshl_add_u32,
  * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's mix, 5 instructions per two MACs) and
  * the LDS gather rate (kinds 1..6: u8 / u16 / b32 reads, lanes inside one
- * 128-element row or scattered).  Launches
+ * 128-element row or scattered, with 64 KB of LDS per workgroup; kinds 21 / 22: the u8 pair
+ * again at the GEMM kernel's own LDS footprint and occupancy, reads software-pipelined).
+ * Kinds 10..15 also leave two 64-bit counts at sink[512..515]: the shader-clock ticks of one
+ * workgroup's loop and the same interval in 100 MHz ticks (their ratio is the clock).  Launches
  * `reps` times on `stream`, timed with HIP events; `sink` is any device buffer
  * of >= 256 floats. */
 int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream, float *sink,
                      double *ms_per_launch, double *ops_per_launch);
+/* The rates that bound products through tables too wide for the LDS (mantissa widths 8..11,
+ * rows of 4 KB in device memory): kind 0 = one 2-byte global gather per product, all lanes of a
+ * wavefront inside one random row; 1 = whole random rows pulled into LDS by direct
+ * global-to-LDS loads (bytes); 2 = 16-bit LDS gathers with the lanes scattered over 4 KB rows;
+ * 3 = 1 and 2 overlapped in the shape of the row-staged GEMM (64 KB of rows per 65536
+ * products).  `table` is a device buffer of table_bytes >= 8 KB, 16-byte aligned; workgroups
+ * have 1024 threads; ops_per_launch counts products (bytes for kind 1). */
+int amsim_microbench_wide(int kind, int blocks, int iters, int reps, void *stream, const void *table,
+                          size_t table_bytes, float *sink, double *ms_per_launch, double *ops_per_launch);
 
 /* Plain copy kernel of known size (reads 4n bytes, writes 4n bytes; n % 4 == 0,
  * 16-byte aligned buffers): the reference point that hardware traffic counters
