@@ -4,6 +4,7 @@
 #include "amsim_internal.h"
 
 #include <algorithm>
+#include <mutex>
 #include <string>
 
 namespace amsim {
@@ -191,6 +192,55 @@ int amsim_convam_bias_act_f32(amsim_lut_t lut, const float *input_data, float *o
     d.bias_j = bias; d.act = activation;
     d.lane_first = true;  // P(input, filter)
     return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+// ---- allocation-free forward convolution ---------------------------------------------
+// The scratch of amsim_convam_noalloc_f32: part of the device image, so it exists on every GPU
+// the code object is loaded on, at an address of its own there.  In host code the array's name
+// is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+static __device__ __align__(256) unsigned char noalloc_scratch[AMSIM_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int NOALLOC_MAX_DEVICES = 64;
+std::mutex g_noalloc_lock;
+void *g_noalloc_ptr[NOALLOC_MAX_DEVICES];  // device address of noalloc_scratch, per device (null = not asked yet)
+
+// address of the scratch array on the current device, looked up once per device
+int noalloc_scratch_ptr(void **out)
+{
+    int dev = 0;
+    AMSIM_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return fail(AMSIM_ERR_UNSUPPORTED, "device index out of range");
+    std::lock_guard<std::mutex> guard(g_noalloc_lock);
+    if (g_noalloc_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        AMSIM_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(noalloc_scratch)));
+        if (p == nullptr || ((uintptr_t)p & 255)) return fail(AMSIM_ERR_HIP, "scratch symbol has no usable device address");
+        g_noalloc_ptr[dev] = p;
+    }
+    *out = g_noalloc_ptr[dev];
+    return AMSIM_OK;
+}
+}  // namespace
+
+int amsim_convam_noalloc_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
+                             int out_cols, int out_depth, int stride_cols, int stride_rows, int filter_left_offset,
+                             int filter_top_offset, int filter_rows, int filter_cols, int in_depth, int input_cols,
+                             int input_rows, const float *filter, void *stream)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (batch < 0 || out_rows < 0 || out_cols < 0 || out_depth < 0 || filter_rows < 0 || filter_cols < 0 || in_depth < 0)
+        return fail(AMSIM_ERR_INVALID, "bad convolution geometry");
+    const size_t need = amsim_convam_workspace_bytes(batch, out_rows, out_cols, out_depth, filter_rows, filter_cols, in_depth);
+    if (need > AMSIM_NOALLOC_SCRATCH_BYTES)
+        return fail(AMSIM_ERR_UNSUPPORTED, "problem needs " + std::to_string(need) + " bytes of scratch, the allocation-free "
+                                           "entry point holds " + std::to_string(AMSIM_NOALLOC_SCRATCH_BYTES));
+    void *scratch = nullptr;
+    if (const int rc = noalloc_scratch_ptr(&scratch)) return rc;
+    return amsim_convam_bias_act_f32(lut, input_data, output_data, batch, out_rows, out_cols, out_depth, stride_cols,
+                                     stride_rows, filter_left_offset, filter_top_offset, filter_rows, filter_cols,
+                                     in_depth, input_cols, input_rows, filter, nullptr, AMSIM_ACT_NONE, scratch,
+                                     AMSIM_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 // ---- grad-input ----------------------------------------------------------------------

@@ -132,6 +132,23 @@ int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_dat
                      int input_rows, const float *filter, void *workspace, size_t workspace_bytes,
                      void *stream);
 
+/* amsim_convam_f32 for callers that cannot allocate device memory or bring a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The call takes its scratch (pre-decoded filter, partial sums of
+ * split reductions) from a buffer of AMSIM_NOALLOC_SCRATCH_BYTES that is part of the library's
+ * device image -- every GPU the library runs on holds it from the first call until the process
+ * ends -- and calls no hipMalloc, hipFree or other allocating routine.  Problems whose
+ * amsim_convam_workspace_bytes exceeds that size are refused with AMSIM_ERR_UNSUPPORTED.
+ * Results are bit-identical to amsim_convam_f32 on the same inputs.  All calls on one GPU share
+ * the one buffer: calls that may overlap there (different streams or threads) race; issue them
+ * on one stream, or order them with events.  Nothing in the buffer needs to start at zero (each
+ * call writes what it later reads). */
+#define AMSIM_NOALLOC_SCRATCH_BYTES ((size_t)32 << 20)
+int amsim_convam_noalloc_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
+                             int out_cols, int out_depth, int stride_cols, int stride_rows, int filter_left_offset,
+                             int filter_top_offset, int filter_rows, int filter_cols, int in_depth, int input_cols,
+                             int input_rows, const float *filter, void *stream);
+
 /* The same with the layer's epilogue fused into the store: output = act(conv + bias[out_depth]).
  * Replaces Convam followed by BiasAdd and the activation op in AMConv2D.call
  * (python/keras/layers/am_convolutional.py:248-276); bias may be NULL.  Bit-identical to the
