@@ -44,14 +44,19 @@ struct GemmCall {
     int act = AMSIM_ACT_NONE;
 };
 
-GemmDesc describe(const GemmCall &g)
+// wide_table: the LUT is too wide for the LDS (mantissa width above 7).  The row-staged engine that
+// serves such tables wants as many rows over the lanes as it can get, so the longer of M and N
+// goes there when that makes the problem eligible for it.
+GemmDesc describe(const GemmCall &g, bool wide_table)
 {
     GemmDesc d;
     d.K = g.K;
     d.batch = (int)g.batch;
     d.out = g.C;
     d.out_batch_stride = g.strideC;
-    if (lanes_along_m(g.M, g.N, g.K)) {
+    bool along_m = lanes_along_m(g.M, g.N, g.K);
+    if (wide_table && wide_shape_eligible(std::max(g.M, g.N), (int)g.batch)) along_m = g.M >= g.N;
+    if (along_m) {
         d.R = g.M; d.J = g.N;
         d.p.kind = P_DENSE; d.p.base = g.A; d.p.batch_stride = g.strideA;
         d.p.sr = g.transA ? 1 : g.lda; d.p.sk = g.transA ? g.lda : 1;
@@ -88,14 +93,16 @@ int gemm_call(amsim_lut_t lut, const GemmCall &g, void *ws, size_t ws_bytes, voi
     const int64_t min_lda = g.transA ? g.M : g.K, min_ldb = g.transB ? g.K : g.N;
     if (g.lda < min_lda || g.ldb < min_ldb || g.ldc < g.N)
         return fail(AMSIM_ERR_INVALID, "leading dimension smaller than the row length");
-    return run_gemm(lut->l, describe(g), ws, ws_bytes, static_cast<hipStream_t>(stream));
+    return run_gemm(lut->l, describe(g, lut->l.m > 7), ws, ws_bytes, static_cast<hipStream_t>(stream));
 }
 
 size_t gemm_ws(const GemmCall &g)
 {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) return 0;
-    GemmDesc d = describe(g);
-    return gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
+    // valid for any table: the orientation (and with it the engine) depends on the table's width
+    const GemmDesc d = describe(g, false), w = describe(g, true);
+    return std::max(gemm_workspace_bytes_any_lut(d.R, d.J, d.K, d.batch, d.q.batches),
+                    gemm_workspace_bytes_any_lut(w.R, w.J, w.K, w.batch, w.q.batches));
 }
 
 bool fits_int32(int64_t elements) { return elements < (1ll << 31); }
@@ -128,7 +135,7 @@ int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K
 {
     if (!info || M <= 0 || N <= 0 || K <= 0 || batch <= 0) return fail(AMSIM_ERR_INVALID, "bad plan query");
     GemmCall g{transA, transB, 0, M, N, K, nullptr, transA ? M : K, nullptr, transB ? K : N, nullptr, N, batch, 1, 1, 1};
-    const GemmDesc d = describe(g);
+    const GemmDesc d = describe(g, false);
     // contiguous, aligned operands assumed (the float4-staged kernel variants)
     gemm_plan_info(d.R, d.J, d.K, d.batch, d.q.batches, true, d.p.sk == 1 && d.p.sr != 1 ? 6 : 5, info);
     return AMSIM_OK;

@@ -33,57 +33,19 @@
 //     bit-exact everywhere without taxing the fast path.
 #include "amsim_internal.h"
 #include "amsim_device.h"
+#include "amsim_gemm_common.h"
 
 #include <algorithm>
 #include <atomic>
 
 namespace amsim {
 
-constexpr int KC = 32;        // reduction depth of one staged chunk
-constexpr int KG = 4;         // reduction rows handled per scalar-load batch
-constexpr int NG = KC / KG;
-constexpr int QT = 16;        // columns per tile of the pre-decoded uniform operand
-constexpr int WG_THREADS = 256;
-constexpr int LUT_LDS_BYTES = 16384 + 128;   // 2^(2m) entries + one all-zero row of 2^m entries (m <= 7)
-constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels are compiled for
-constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
-constexpr double MACS_PER_CU_S = 13.0e12 / 256;  // planner's price of a MAC: what one compute unit sustains
-constexpr double PARTIAL_BYTES_PER_S = 3.0e12;   // planner's price of writing + re-reading partial sums
-
 static std::atomic<int> g_split_k{1};
-
-typedef const __attribute__((address_space(4))) uint32_t *cq1_t;
-typedef const __attribute__((address_space(4))) uint64_t *cq2_t;
 
 // staging modes of the lane operand
 enum { STAGE_R = 0,   // threads run along r, one element each (source contiguous in r)
        STAGE_K = 1,   // threads run along k, one element each
        STAGE_K4 = 2 };// threads run along k, four consecutive k per 16-byte load
-
-// Output epilogue shared by the main kernel and the split reduction: bias add, then
-// the activation.  ReLU keeps NaN and the sign of a negative zero (x < 0 ? 0 : x).
-struct Epilogue {
-    const float *bias_j, *bias_r;
-    int act;
-    OutMap omap;
-};
-// element offset of output row r (before the column term)
-__device__ __forceinline__ int64_t out_row_offset(const OutMap &m, int64_t r, int64_t so_r)
-{
-    if (!m.enabled) return r * so_r;
-    const int x = (int)(r % m.GW);
-    const int64_t t = r / m.GW;
-    const int y = (int)(t % m.GH);
-    const int64_t b = t / m.GH;
-    return ((b * m.H + (y * m.sy + m.oy)) * m.W + (x * m.sx + m.ox)) * so_r;
-}
-__device__ __forceinline__ float apply_epilogue(const Epilogue &e, float v, int64_t r, int64_t j)
-{
-    if (e.bias_j) v += e.bias_j[j];
-    if (e.bias_r) v += e.bias_r[r];
-    if (e.act == AMSIM_ACT_RELU) v = v < 0.0f ? 0.0f : v;
-    return v;
-}
 
 struct KArgs {
     PDesc p;
@@ -119,27 +81,6 @@ struct KArgs {
 // ---------------------------------------------------------------------------
 // uniform-operand pre-pass
 // ---------------------------------------------------------------------------
-struct QArgs {
-    QDesc q;
-    int64_t K, J;
-    int Jp, nchunks, m;
-    uint32_t *qw;
-    uint32_t *qflags;
-    QDesc *qdesc_out;
-};
-
-// raw bits of uniform-operand element (k, j) of batch item `base`; zero outside K x J
-// (k < 2^31 and j < 2^24 on every path that gets here)
-template <typename QD>
-__device__ __forceinline__ uint32_t q_raw_bits(const QD &q, const float *base, uint32_t K, uint32_t J, uint32_t k, uint32_t j)
-{
-    if (k >= K || j >= J) return 0u;
-    if (q.kind == Q_DENSE) return f2u(base[(int64_t)k * q.sk + (int64_t)j * q.sj]);
-    const uint32_t oc = k % (uint32_t)q.OC, t = k / (uint32_t)q.OC;
-    const int fx = q.fx0 + (int)(t % (uint32_t)q.TW) * q.fsx, fy = q.fy0 + (int)(t / (uint32_t)q.TW) * q.fsy;
-    return f2u(base[(((int64_t)(q.KH - 1 - fy) * q.KW + (q.KW - 1 - fx)) * q.IC + j) * q.OC + oc]);
-}
-
 // One wavefront per (32-row chunk, 16-column tile): decodes the tile, writes it
 // in the tile-major layout the main kernel streams, and flags the tile-chunk
 // if it holds an operand the fast product path cannot take.  blockIdx.x runs over
@@ -175,6 +116,16 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
     }
     const int any = __any(unsafe);
     if (lane == 0) a.qflags[((size_t)qb * ntiles + jt) * a.nchunks + ch] = (uint32_t)any;
+}
+
+int launch_q_prepass(const QArgs &qa, int q_batches, hipStream_t stream)
+{
+    if (q_batches > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
+    const int64_t wgs = (int64_t)qa.nchunks * ((qa.Jp / QT + 3) / 4);
+    if (wgs >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "uniform operand exceeds the grid limit");
+    q_prepass_kernel<<<dim3((unsigned)wgs, (unsigned)q_batches), WG_THREADS, 0, stream>>>(qa);
+    AMSIM_HIP_CHECK(hipGetLastError());
+    return AMSIM_OK;
 }
 
 // ---------------------------------------------------------------------------
@@ -956,6 +907,20 @@ size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
     return need;
 }
 
+// bytes of the unsplit plan: the pre-decoded uniform operand, its flags and its descriptor
+static size_t unsplit_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
+{
+    return make_plan(R, J, K, batch, q_batches, false, WAVES_PER_SIMD).total;
+}
+
+size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
+{
+    size_t need = gemm_workspace_bytes(R, J, K, batch, q_batches);
+    if (need && wide_shape_eligible(R, batch))
+        need = std::max(need, unsplit_bytes(R, J, K, batch, q_batches) + wide_workspace_bytes(R, K));
+    return need;
+}
+
 // what the planner decides for a problem: {TN, WR, nsplit, chunks per split, rows of the main
 // part, tail nsplit, tail chunks per split, chunks} (for tests and tuning)
 void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int64_t info[8])
@@ -1036,6 +1001,23 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     }
     if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
+    if (wide_eligible(lut.m, d)) {
+        // tables too wide for the LDS: the row-staged engine, if the workspace also holds the
+        // transposed lane operand (else the global-gather variant below does the job, slowly)
+        const Plan pq = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, false, WAVES_PER_SIMD);
+        if (workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
+            workspace_bytes >= pq.total + wide_workspace_bytes(d.R, d.K)) {
+            uint8_t *ws = static_cast<uint8_t *>(workspace);
+            QArgs qa{};
+            qa.q = d.q;
+            qa.K = d.K; qa.J = d.J; qa.Jp = pq.Jp; qa.nchunks = pq.nchunks; qa.m = lut.m;
+            qa.qw = reinterpret_cast<uint32_t *>(ws + pq.off_qw);
+            qa.qflags = reinterpret_cast<uint32_t *>(ws + pq.off_flags);
+            qa.qdesc_out = reinterpret_cast<QDesc *>(ws + pq.off_qdesc);
+            if (const int rc = launch_q_prepass(qa, d.q.batches, stream)) return rc;
+            return run_gemm_wide(lut, d, WideQ{qa.qw, qa.qflags, qa.qdesc_out, pq.Jp, pq.nchunks}, ws + pq.total, stream);
+        }
+    }
     // the handle's own setting wins over the process default (read once per call)
     const bool may_split = (lut.split_k >= 0 ? lut.split_k != 0 : g_split_k.load() != 0) && !d.no_split;
     const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, may_split, waves64_of(d.p, d.K));
@@ -1052,11 +1034,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     qa.qw = reinterpret_cast<uint32_t *>(ws + pl.off_qw);
     qa.qflags = reinterpret_cast<uint32_t *>(ws + pl.off_flags);
     qa.qdesc_out = reinterpret_cast<QDesc *>(ws + pl.off_qdesc);
-    if (d.q.batches > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
-    const int64_t prepass_wgs = (int64_t)pl.nchunks * ((pl.Jp / QT + 3) / 4);
-    if (prepass_wgs >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "uniform operand exceeds the grid limit");
-    q_prepass_kernel<<<dim3((unsigned)prepass_wgs, (unsigned)d.q.batches), WG_THREADS, 0, stream>>>(qa);
-    AMSIM_HIP_CHECK(hipGetLastError());
+    if (const int rc = launch_q_prepass(qa, d.q.batches, stream)) return rc;
 
     KArgs ka{};
     ka.p = d.p;

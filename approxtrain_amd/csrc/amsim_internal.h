@@ -119,6 +119,25 @@ size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
 void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int64_t info[8]);
 int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream);
 
+// ---- the row-staged engine for tables too wide for the LDS (mantissa widths 8..11) ----------
+// Serves dense, unbatched problems with at least WIDE_MIN_ROWS rows when the caller's workspace
+// also holds the transposed lane operand (wide_workspace_bytes on top of the unsplit plan);
+// everything else with such tables runs on the LDS-table engine's global-gather variant.
+constexpr int64_t WIDE_MIN_ROWS = 1024;
+struct WideQ {
+    const uint32_t *qw;
+    const uint32_t *qflags;
+    const QDesc *qdesc;
+    int Jp, nchunks;
+};
+bool wide_shape_eligible(int64_t R, int batch);
+bool wide_eligible(int m, const GemmDesc &d);
+size_t wide_workspace_bytes(int64_t R, int64_t K);
+int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, hipStream_t stream);
+// workspace that serves a dense problem with any table: the larger of gemm_workspace_bytes and
+// what the row-staged engine needs
+size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
+
 int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream);
 
 // Strided grad-input runs one sub-problem per residue class of the input pixels, each over the

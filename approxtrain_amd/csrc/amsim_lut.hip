@@ -92,7 +92,8 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
         if ((rc = upload(&l.img_ab, ab)) != AMSIM_OK) return rc;
         if ((rc = upload(&l.img_ba, ba)) != AMSIM_OK) return rc;
     } else {
-        std::vector<uint16_t> ab(total + n, 0), ba(total + n, 0);  // + the all-zero row
+        // + the all-zero row, + 4 KB: the row-staged GEMM copies whole KBs from a row's start
+        std::vector<uint16_t> ab(total + n + 2048, 0), ba(total + n + 2048, 0);
         for (size_t i = 0; i < n; ++i)
             for (size_t j = 0; j < n; ++j) {
                 const uint16_t b = (uint16_t)((carry[i * n + j] << 15) | (mant[i * n + j] << (15 - m)));

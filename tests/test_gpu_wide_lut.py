@@ -1,0 +1,145 @@
+"""Tables too wide for the LDS (mantissa widths 8..11) on the row-staged engine: dense problems
+with at least 1024 rows, through the C ABI, BIT-EQUAL to the CPU oracle (one ascending-k FP32
+chain per output: that engine never splits a reduction).
+
+Parity note: no reference file or functional model exists above width 7.  The tables come from
+the oracle's generator, i.e. from the closed-form rules that reproduce every reference file up to
+width 7; beyond that rule the tables' parity is unpinned.  What these tests pin is that the GPU
+multiplies and accumulates through whatever table it is given exactly like the oracle's loop nest
+(cuda/gemm.cu:17-58 with the lookup of lut/AMsimulator.inl:18-23)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu
+from tests.gpu_util import dev, host
+from tests.util import same_bits_or_both_nan
+
+pytestmark = pytest.mark.gpu
+
+
+def _legacy(img):
+    return (((img >> 23) << 31) | (img & 0x7fffff)).astype(np.uint32)
+
+
+@pytest.fixture(scope="module")
+def luts():
+    from approxtrain_amd import ApproxMulLut
+    cache = {}
+
+    def get(kind, m):
+        if (kind, m) not in cache:
+            img = cpu.lutgen32(kind, m)
+            cache[(kind, m)] = (ApproxMulLut.from_entries(_legacy(img), m), img)
+        return cache[(kind, m)]
+    return get
+
+
+def _ops(rng, M, N, K, ta, tb):
+    A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+    B = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    A[rng.random(A.shape) < 0.1] = 0.0
+    B[rng.random(B.shape) < 0.05] = 0.0
+    return A, B
+
+
+@pytest.mark.parametrize("kind,m", [("MBM", 11), ("MIT", 11), ("MBM", 10), ("MIT", 9), ("MBM", 8)])
+@pytest.mark.parametrize("M,N,K,ta,tb", [(1100, 37, 70, 0, 0), (40, 2100, 64, 0, 0), (4200, 16, 33, 1, 0),
+                                         (1030, 50, 96, 0, 1), (24, 1500, 40, 1, 1)])
+def test_row_staged_gemm_bit_equal_to_oracle(luts, kind, m, M, N, K, ta, tb):
+    from approxtrain_amd import functors
+    lut, img = luts(kind, m)
+    rng = np.random.default_rng(1000 * m + M + N + K + 2 * ta + tb)
+    A, B = _ops(rng, M, N, K, ta, tb)
+    got = host(functors.gemm(lut, dev(A), dev(B), trans_a=bool(ta), trans_b=bool(tb)))
+    want = cpu.gemm(img, m, A, B, transA=ta, transB=tb)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("m", [11, 8])
+def test_row_staged_gemm_full_domain_operands(luts, m):
+    """Subnormals, infinities, NaN, huge and tiny magnitudes in either operand flag their
+    32-deep chunk, which then takes the full-domain product; NaNs compare as a class."""
+    from approxtrain_amd import functors
+    lut, img = luts("MBM", m)
+    rng = np.random.default_rng(5 + m)
+    M, N, K = 1300, 40, 100
+    A, B = _ops(rng, M, N, K, 0, 0)
+    specials = np.array([1e-40, -1e-42, np.inf, -np.inf, np.nan, 3e38, -1e-38, 2.0 ** -70, 2.0 ** 70], np.float32)
+    for s in specials:
+        A[rng.integers(M), rng.integers(K)] = s
+        B[rng.integers(K), rng.integers(N)] = s
+    A[700, 40:72] = 2.0 ** 100   # a chunk flagged by the lane operand only
+    B[64:96, 7] = 2.0 ** -100    # a chunk flagged by the uniform operand only
+    got = host(functors.gemm(lut, dev(A), dev(B)))
+    want = cpu.gemm(img, m, A, B)
+    assert same_bits_or_both_nan(got, want).all()
+    assert np.isnan(want).any() and np.isfinite(want).any()
+
+
+def test_row_staged_gemm_operand_order_with_asymmetric_table(luts):
+    """A table whose entry depends on which operand indexes its row: both LUT orientations
+    (the two transposed device images) and the swap flag must agree with the oracle."""
+    from approxtrain_amd import ApproxMulLut, functors
+    m = 8
+    n = 1 << m
+    i, j = np.meshgrid(np.arange(n, dtype=np.uint32), np.arange(n, dtype=np.uint32), indexing="ij")
+    mant = (i * 3 + j * 5 + 1) % n
+    img = (((i > j).astype(np.uint32) << 23) | (mant << (23 - m))).astype(np.uint32).ravel()
+    lut = ApproxMulLut.from_entries(_legacy(img), m)
+    rng = np.random.default_rng(8)
+    A, B = _ops(rng, 1200, 30, 48, 0, 0)
+    for swap in (False, True):
+        got = host(functors.gemm(lut, dev(A), dev(B), swap_operands=swap))
+        want = cpu.gemm(img, m, A, B, swap=swap)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # rows over N: the other device image serves the same product
+    A2, B2 = _ops(rng, 20, 1400, 48, 0, 0)
+    for swap in (False, True):
+        got = host(functors.gemm(lut, dev(A2), dev(B2), swap_operands=swap))
+        want = cpu.gemm(img, m, A2, B2, swap=swap)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dense_layer_with_fused_epilogue_on_row_staged_engine(luts):
+    from approxtrain_amd import functors
+    lut, img = luts("MIT", 11)
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((1500, 40)).astype(np.float32)
+    w = rng.standard_normal((40, 24)).astype(np.float32)
+    b = rng.standard_normal(24).astype(np.float32)
+    got = host(functors.denseam(lut, dev(x), dev(w), bias=dev(b), activation="relu"))
+    y = cpu.dense_fwd(img, 11, x, w) + b
+    want = np.where(y < 0, np.float32(0), y).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_smaller_workspace_falls_back_to_global_gathers(luts):
+    """The LUT-less workspace query covers the row-staged engine; a caller that brings only what
+    the global-gather variant needs still gets the same bits."""
+    import approxtrain_amd
+    from approxtrain_amd._lib import check
+    lib = approxtrain_amd.load_library()
+    lut, img = luts("MBM", 11)
+    rng = np.random.default_rng(13)
+    M, N, K = 1100, 20, 64
+    A, B = _ops(rng, M, N, K, 0, 0)
+    Ad, Bd = dev(A), dev(B)
+    full = lib.amsim_gemm_workspace_bytes(0, 0, M, N, K, 1)
+    assert full > 4 * M * K   # holds the transposed lane operand
+    small = 512 * 1024
+    outs = []
+    for nbytes in (full, small):
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device="cuda")
+        wsp = C.c_void_p(ws.data_ptr() + (-ws.data_ptr()) % 256)
+        out = torch.empty((M, N), device="cuda")
+        lib.amsim_lut_set_split_k(lut.handle, 0)
+        check(lib.amsim_gemm_f32(lut.handle, 0, 0, 0, M, N, K, C.c_void_p(Ad.data_ptr()), K, C.c_void_p(Bd.data_ptr()), N,
+                                 C.c_void_p(out.data_ptr()), N, 1, 0, 0, 0, wsp, nbytes, None))
+        lib.amsim_lut_set_split_k(lut.handle, -1)
+        outs.append(host(out))
+    want = cpu.gemm(img, 11, A, B)
+    assert np.array_equal(outs[0].view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(outs[1].view(np.uint32), want.view(np.uint32))
