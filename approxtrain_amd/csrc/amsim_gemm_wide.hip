@@ -8,11 +8,12 @@
 // 2^m-entry row of the table (the one q(k, j)'s mantissa selects; 4 KB at width 11): a workgroup
 // that owns many rows r pulls that row into LDS once and lets all its rows gather from there.
 //
-//   * one workgroup = 1024 threads = 4096 rows (4 per thread) x 16 columns, the whole reduction;
-//   * per reduction step k ("stage") the 16 wavefronts copy the 16 table rows of q(k+1, j0..j0+15)
-//     into one half of a 128 KB LDS buffer with direct global-to-LDS loads (no registers), while
-//     every thread gathers its 4 x 16 entries of stage k from the other half: 64 KB pulled in per
-//     65 536 products = 1 byte per product;
+//   * one workgroup = 512 threads = 4096 rows (8 per thread) x 8 columns, the whole reduction; two
+//     workgroups share a compute unit;
+//   * per reduction step k ("stage") the 8 wavefronts copy the 8 table rows of q(k+1, j0..j0+7)
+//     into one half of a 64 KB LDS buffer with direct global-to-LDS loads (no registers), while
+//     every thread gathers its 8 x 8 entries of stage k from the other half: 32 KB pulled in per
+//     32 768 products = 1 byte per product;
 //   * the lane operand p is transposed once per call into [k][row] order in the workspace
 //     (raw bits, zero-padded), so a thread's operands arrive by fully coalesced 4-byte loads,
 //     prefetched one stage ahead, and never touch the LDS;
@@ -31,12 +32,13 @@ namespace amsim {
 
 namespace {
 
-constexpr int WIDE_THREADS = 1024;
-constexpr int WIDE_RPT = 4;                       // rows per thread
-constexpr int WIDE_TILE_ROWS = WIDE_THREADS * WIDE_RPT;
-constexpr int WIDE_TN = QT;                       // columns per workgroup = one tile of the pre-decoded operand
+// A workgroup is 512 threads = 8 wavefronts (one per staged table row) on 4096 rows x 8 columns, and
+// two of them share a compute unit: while one waits at its stage barrier the other gathers (measured
+// 4.7 TMAC/s against 4.45 for one 1024-thread workgroup on 16 columns).
+constexpr int WIDE_TILE_ROWS = 4096;              // rows per workgroup
+constexpr int WIDE_TN = 8;                        // columns per workgroup: half a tile of the pre-decoded operand
+constexpr int WIDE_THREADS = WIDE_TN * 64;
 constexpr int WIDE_SLOT_BYTES = 4096;             // LDS bytes reserved per staged table row (2^11 entries x 2)
-constexpr int WIDE_BUF_BYTES = WIDE_TN * WIDE_SLOT_BYTES;
 constexpr int PT_ROWS = 64;                       // rows per workgroup of the transposing pre-pass
 
 struct PTArgs {
@@ -86,33 +88,24 @@ __device__ __forceinline__ uint32_t lds_addr(const void *p)
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
 
-// The 16 entries at addr + j * 4 KB (one per staged table row), issued back to back and waited for
-// together.  Written as one block so that the 16 gathers of a row group stay 16 registers wide (left
-// to itself the scheduler hoists all 64 of a stage and spills accumulators), and so that the compiler
+// The 8 entries at addr + j * 4 KB (one per staged table row), issued back to back and waited for
+// together.  Written as one block so that the gathers of a row group stay 8 registers wide (left to
+// itself the scheduler hoists all 64 of a stage and spills accumulators), and so that the compiler
 // does not order them behind the direct-to-LDS copies in flight for the next stage, which write the
 // other half of the buffer.
-__device__ __forceinline__ void gather16(uint32_t addr, uint32_t (&e)[16])
+__device__ __forceinline__ void gather8(uint32_t addr, uint32_t (&e)[8])
 {
     asm volatile(
-        "ds_read_u16 %0, %16\n\t"
-        "ds_read_u16 %1, %16 offset:4096\n\t"
-        "ds_read_u16 %2, %16 offset:8192\n\t"
-        "ds_read_u16 %3, %16 offset:12288\n\t"
-        "ds_read_u16 %4, %16 offset:16384\n\t"
-        "ds_read_u16 %5, %16 offset:20480\n\t"
-        "ds_read_u16 %6, %16 offset:24576\n\t"
-        "ds_read_u16 %7, %16 offset:28672\n\t"
-        "ds_read_u16 %8, %16 offset:32768\n\t"
-        "ds_read_u16 %9, %16 offset:36864\n\t"
-        "ds_read_u16 %10, %16 offset:40960\n\t"
-        "ds_read_u16 %11, %16 offset:45056\n\t"
-        "ds_read_u16 %12, %16 offset:49152\n\t"
-        "ds_read_u16 %13, %16 offset:53248\n\t"
-        "ds_read_u16 %14, %16 offset:57344\n\t"
-        "ds_read_u16 %15, %16 offset:61440\n\t"
+        "ds_read_u16 %0, %8\n\t"
+        "ds_read_u16 %1, %8 offset:4096\n\t"
+        "ds_read_u16 %2, %8 offset:8192\n\t"
+        "ds_read_u16 %3, %8 offset:12288\n\t"
+        "ds_read_u16 %4, %8 offset:16384\n\t"
+        "ds_read_u16 %5, %8 offset:20480\n\t"
+        "ds_read_u16 %6, %8 offset:24576\n\t"
+        "ds_read_u16 %7, %8 offset:28672\n\t"
         "s_waitcnt lgkmcnt(0)"
-        : "=&v"(e[0]), "=&v"(e[1]), "=&v"(e[2]), "=&v"(e[3]), "=&v"(e[4]), "=&v"(e[5]), "=&v"(e[6]), "=&v"(e[7]),
-          "=&v"(e[8]), "=&v"(e[9]), "=&v"(e[10]), "=&v"(e[11]), "=&v"(e[12]), "=&v"(e[13]), "=&v"(e[14]), "=&v"(e[15])
+        : "=&v"(e[0]), "=&v"(e[1]), "=&v"(e[2]), "=&v"(e[3]), "=&v"(e[4]), "=&v"(e[5]), "=&v"(e[6]), "=&v"(e[7])
         : "v"(addr)
         : "memory");
 }
@@ -137,9 +130,11 @@ struct WArgs {
 // PARTS: KB of a table row copied per stage and slot (4 at width 11, 2 at width 10, 1 below: the copy
 // of a narrower row runs on into the rows behind it, which the image's padding keeps in bounds).
 template <int PARTS>
-__global__ __launch_bounds__(WIDE_THREADS) void lutgemm_wide_kernel(WArgs a)
+__global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
 {
-    // Two halves of 16 slots x 4 KB, as two objects: the compiler then knows that the direct-to-LDS
+    constexpr int WIDE_RPT = WIDE_TILE_ROWS / WIDE_THREADS;
+    constexpr int WIDE_BUF_BYTES = WIDE_TN * WIDE_SLOT_BYTES;
+    // Two halves of 8 slots x 4 KB, as two objects: the compiler then knows that the direct-to-LDS
     // copies into one half do not alias the gathers from the other, and does not make the gathers
     // wait for the copies.
     __shared__ __align__(16) uint8_t rows_a[WIDE_BUF_BYTES];
@@ -159,11 +154,12 @@ __global__ __launch_bounds__(WIDE_THREADS) void lutgemm_wide_kernel(WArgs a)
     }
     const int64_t row0 = (int64_t)bx * WIDE_TILE_ROWS;
     const int j0 = by * WIDE_TN;
+    constexpr int STRIPS_PER_TILE = QT / WIDE_TN;
     const int m = a.m, mshift = 23 - m;
     const uint32_t mmask = (1u << m) - 1u;
     const int Kp = a.nchunks * KC;
-    const cq1_t qtile = (cq1_t)(uintptr_t)(a.qw + (size_t)by * Kp * QT);
-    const cq1_t qfl = (cq1_t)(uintptr_t)(a.qflags + (size_t)by * a.nchunks);
+    const cq1_t qtile = (cq1_t)(uintptr_t)(a.qw + (size_t)(by / STRIPS_PER_TILE) * Kp * QT + (by % STRIPS_PER_TILE) * WIDE_TN);
+    const cq1_t qfl = (cq1_t)(uintptr_t)(a.qflags + (size_t)(by / STRIPS_PER_TILE) * a.nchunks);
     const uint32_t *pcol = a.pt + row0 + tid;
     const int64_t G = a.Rp / PT_ROWS;
     float acc[WIDE_RPT][WIDE_TN];
@@ -216,7 +212,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void lutgemm_wide_kernel(WArgs a)
                     const float ta = u2f(pc[rr] & 0xff800000u);
                     const uint32_t off = ((pc[rr] >> mshift) & mmask) << 1;
                     uint32_t e[WIDE_TN];
-                    gather16(lds_addr(cur) + off, e);
+                    gather8(lds_addr(cur) + off, e);
 #pragma unroll
                     for (int j = 0; j < WIDE_TN; ++j)
                         // (entry << 8) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly
@@ -340,7 +336,7 @@ int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_
     wa.vec_store = (d.so_j == 1 && d.so_r % 4 == 0 && ((uintptr_t)d.out & 15) == 0) ? 1 : 0;
     wa.ep = Epilogue{d.bias_j, d.bias_r, d.act, d.omap};
     wa.X = (unsigned)(Rp / WIDE_TILE_ROWS);
-    wa.Y = (unsigned)(q.Jp / QT);
+    wa.Y = (unsigned)(q.Jp / WIDE_TN);
     const int64_t total = (int64_t)wa.X * wa.Y;
     if (total >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "workgroup count exceeds the grid limit");
     if (lut.m >= 11) lutgemm_wide_kernel<4><<<dim3((unsigned)total), WIDE_THREADS, 0, stream>>>(wa);

@@ -104,13 +104,20 @@ def test_cfg3_resnet50_3x3_full_size_filter_grad(cfg3):
     assert_close_sum_abs(full, parts, s_full, REL)
 
 
-@pytest.mark.parametrize("kind,m", [("MBM", 7), ("MIT", 5), ("MBM", 1)])
+@pytest.mark.parametrize("kind,m", [(k, m) for k in ("MBM", "MIT") for m in (1, 3, 5, 7, 11)])
 def test_cfg4_square_gemm_4096_sampled_against_oracle(kind, m):
-    """C = A.B, dA = dC.B^T, dB = A^T.dC at 4096^3: 48 x 48 sampled outputs of
-    each are recomputed by the oracle (full-length 4096-term reductions)."""
+    """C = A.B, dA = dC.B^T, dB = A^T.dC at 4096^3 for every table of the sweep: 48 x 48 sampled
+    outputs of each are recomputed by the oracle (full-length 4096-term reductions).  The width-11
+    tables come from the generator: no reference file or model exists above width 7, so their
+    parity is unpinned beyond the closed-form rule that reproduces every reference file; the
+    test pins the multiply-accumulate through the table, not the table."""
     from approxtrain_amd import ApproxMulLut, functors
-    lut = ApproxMulLut.cached(lut_path(kind, m))
-    L = lut32(kind, m)
+    if m <= 7:
+        lut = ApproxMulLut.cached(lut_path(kind, m))
+        L = lut32(kind, m)
+    else:
+        L = cpu.lutgen32(kind, m)
+        lut = ApproxMulLut.from_entries((((L >> 23) << 31) | (L & 0x7fffff)).astype(np.uint32), m)
     n = 4096
     A = np.random.default_rng(12).standard_normal((n, n)).astype(np.float32)
     B = np.random.default_rng(13).standard_normal((n, n)).astype(np.float32)
