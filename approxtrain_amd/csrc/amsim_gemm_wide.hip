@@ -191,82 +191,98 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for (int ch = 0; ch < a.nchunks; ++ch) {
-        // a chunk is flagged by its column tile or by any 64-row group of this row tile
-        const uint32_t pf = a.pflags[(size_t)ch * G + (size_t)bx * (WIDE_TILE_ROWS / PT_ROWS) + lane];
-        const bool unsafe = (qfl[ch] != 0u) | (__any(pf != 0u) != 0);
-        // one stage: copies for stage k + 1 go into `next` while stage k gathers from `cur`
-        auto stage = [&](auto exact_tag, int k, const uint8_t *cur, uint8_t *next) {
-            constexpr bool EXACT = decltype(exact_tag)::value;
-            // (the last stage copies its own rows and operands once more instead of branching: a
-            // straight-line stage keeps the compiler from sinking one stage's FMAs into the next)
-            const int kn = min(k + 1, Kp - 1);
-            fill(kn, next);  // everyone left that half at the barrier that ended the stage before
-            load_p(kn, pn);
-            if constexpr (!EXACT) {
-                uint32_t qt[WIDE_TN];
+    // Is any chunk of this workgroup's tile flagged (by its column tile or by a 64-row group of its
+    // row tile)?  Almost never: then the whole reduction runs the loop nest that holds nothing but
+    // fast stages, whose registers the rare path's state cannot crowd.
+    int tile_flagged = 0;
+    for (int ch = 0; ch < a.nchunks; ++ch) tile_flagged |= (int)qfl[ch];
+    for (int i = tid; i < a.nchunks * (WIDE_TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
+        tile_flagged |= (int)a.pflags[(size_t)(i / (WIDE_TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (WIDE_TILE_ROWS / PT_ROWS) +
+                                     i % (WIDE_TILE_ROWS / PT_ROWS)];
+    tile_flagged = __syncthreads_or(tile_flagged);
+
+    // one stage: copies for stage k + 1 go into `next` while stage k gathers from `cur`
+    auto stage = [&](auto exact_tag, int k, const uint8_t *cur, uint8_t *next) {
+        constexpr bool EXACT = decltype(exact_tag)::value;
+        // (the last stage copies its own rows and operands once more instead of branching: a
+        // straight-line stage keeps the compiler from sinking one stage's FMAs into the next)
+        const int kn = min(k + 1, Kp - 1);
+        fill(kn, next);  // everyone left that half at the barrier that ended the stage before
+        load_p(kn, pn);
+        if constexpr (!EXACT) {
+            uint32_t qt[WIDE_TN];
 #pragma unroll
-                for (int j = 0; j < WIDE_TN; ++j) qt[j] = qtile[k * QT + j] & 0xff800000u;
+            for (int j = 0; j < WIDE_TN; ++j) qt[j] = qtile[k * QT + j] & 0xff800000u;
 #pragma unroll
-                for (int rr = 0; rr < WIDE_RPT; ++rr) {
-                    const float ta = u2f(pc[rr] & 0xff800000u);
-                    const uint32_t off = ((pc[rr] >> mshift) & mmask) << 1;
-                    uint32_t e[WIDE_TN];
-                    gather8(lds_addr(cur) + off, e);
+            for (int rr = 0; rr < WIDE_RPT; ++rr) {
+                const float ta = u2f(pc[rr] & 0xff800000u);
+                const uint32_t off = ((pc[rr] >> mshift) & mmask) << 1;
+                uint32_t e[WIDE_TN];
+                gather8(lds_addr(cur) + off, e);
 #pragma unroll
-                    for (int j = 0; j < WIDE_TN; ++j)
-                        // (entry << 8) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly
-                        acc[rr][j] = __builtin_fmaf(ta, u2f((e[j] << 8) + qt[j]), acc[rr][j]);
-                }
-            } else {
-                // Rare: full-domain product; q's raw bits come from where the operand lies.  The
-                // accumulators take a detour through private memory so that this loop can index them
-                // dynamically (small code, one product at a time) while the fast path keeps them in
-                // registers.
-                const __attribute__((address_space(4))) QDesc &qd = *(const __attribute__((address_space(4))) QDesc *)(uintptr_t)a.qdesc;
-                const float *qsrc = qd.base;
-                float tmp[WIDE_RPT * WIDE_TN];
-                uint32_t praw[WIDE_RPT];
-#pragma unroll
-                for (int rr = 0; rr < WIDE_RPT; ++rr) {
-                    praw[rr] = pc[rr];
-#pragma unroll
-                    for (int j = 0; j < WIDE_TN; ++j) tmp[rr * WIDE_TN + j] = acc[rr][j];
-                }
-#pragma unroll 1
-                for (int idx = 0; idx < WIDE_RPT * WIDE_TN; ++idx) {
-                    const int rr = idx / WIDE_TN, j = idx % WIDE_TN;
-                    const uint32_t raw = praw[rr];
-                    const uint32_t off = ((raw >> mshift) & mmask) << 1;
-                    const uint32_t e16 = (uint32_t)*reinterpret_cast<const uint16_t *>(cur + off + j * WIDE_SLOT_BYTES) << 8;
-                    const uint32_t qr = q_raw_bits(qd, qsrc, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)k, (uint32_t)(j0 + j));
-                    tmp[idx] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
-                }
-#pragma unroll
-                for (int rr = 0; rr < WIDE_RPT; ++rr)
-#pragma unroll
-                    for (int j = 0; j < WIDE_TN; ++j) acc[rr][j] = tmp[rr * WIDE_TN + j];
-            }
-#pragma unroll
-            for (int rr = 0; rr < WIDE_RPT; ++rr) pc[rr] = pn[rr];
-            // my copies for the next stage have landed; after the barrier so have everyone's, and
-            // every wavefront is done gathering from this stage's half
-            __builtin_amdgcn_sched_barrier(0);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-        };
-        // (two loops, so that the rare path's state never meets the fast path's in one loop body)
-        if (!unsafe) {
-#pragma unroll 1
-            for (int kk = 0; kk < KC; kk += 2) {
-                stage(std::false_type{}, ch * KC + kk, rows_a, rows_b);
-                stage(std::false_type{}, ch * KC + kk + 1, rows_b, rows_a);
+                for (int j = 0; j < WIDE_TN; ++j)
+                    // (entry << 8) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly
+                    acc[rr][j] = __builtin_fmaf(ta, u2f((e[j] << 8) + qt[j]), acc[rr][j]);
             }
         } else {
+            // Rare: full-domain product; q's raw bits come from where the operand lies.  The
+            // accumulators take a detour through private memory so that this loop can index them
+            // dynamically (small code, one product at a time) while the fast path keeps them in
+            // registers.
+            const __attribute__((address_space(4))) QDesc &qd = *(const __attribute__((address_space(4))) QDesc *)(uintptr_t)a.qdesc;
+            const float *qsrc = qd.base;
+            float tmp[WIDE_RPT * WIDE_TN];
+            uint32_t praw[WIDE_RPT];
+#pragma unroll
+            for (int rr = 0; rr < WIDE_RPT; ++rr) {
+                praw[rr] = pc[rr];
+#pragma unroll
+                for (int j = 0; j < WIDE_TN; ++j) tmp[rr * WIDE_TN + j] = acc[rr][j];
+            }
 #pragma unroll 1
-            for (int kk = 0; kk < KC; kk += 2) {
-                stage(std::true_type{}, ch * KC + kk, rows_a, rows_b);
-                stage(std::true_type{}, ch * KC + kk + 1, rows_b, rows_a);
+            for (int idx = 0; idx < WIDE_RPT * WIDE_TN; ++idx) {
+                const int rr = idx / WIDE_TN, j = idx % WIDE_TN;
+                const uint32_t raw = praw[rr];
+                const uint32_t off = ((raw >> mshift) & mmask) << 1;
+                const uint32_t e16 = (uint32_t)*reinterpret_cast<const uint16_t *>(cur + off + j * WIDE_SLOT_BYTES) << 8;
+                const uint32_t qr = q_raw_bits(qd, qsrc, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)k, (uint32_t)(j0 + j));
+                tmp[idx] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
+            }
+#pragma unroll
+            for (int rr = 0; rr < WIDE_RPT; ++rr)
+#pragma unroll
+                for (int j = 0; j < WIDE_TN; ++j) acc[rr][j] = tmp[rr * WIDE_TN + j];
+        }
+#pragma unroll
+        for (int rr = 0; rr < WIDE_RPT; ++rr) pc[rr] = pn[rr];
+        // my copies for the next stage have landed; after the barrier so have everyone's, and
+        // every wavefront is done gathering from this stage's half
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+    if (!tile_flagged) {
+#pragma unroll 1
+        for (int k = 0; k < Kp; k += 2) {
+            stage(std::false_type{}, k, rows_a, rows_b);
+            stage(std::false_type{}, k + 1, rows_b, rows_a);
+        }
+    } else {
+        for (int ch = 0; ch < a.nchunks; ++ch) {
+            const uint32_t pf = a.pflags[(size_t)ch * G + (size_t)bx * (WIDE_TILE_ROWS / PT_ROWS) + lane];
+            const bool unsafe = (qfl[ch] != 0u) | (__any(pf != 0u) != 0);
+            if (!unsafe) {
+#pragma unroll 1
+                for (int kk = 0; kk < KC; kk += 2) {
+                    stage(std::false_type{}, ch * KC + kk, rows_a, rows_b);
+                    stage(std::false_type{}, ch * KC + kk + 1, rows_b, rows_a);
+                }
+            } else {
+#pragma unroll 1
+                for (int kk = 0; kk < KC; kk += 2) {
+                    stage(std::true_type{}, ch * KC + kk, rows_a, rows_b);
+                    stage(std::true_type{}, ch * KC + kk + 1, rows_b, rows_a);
+                }
             }
         }
     }
