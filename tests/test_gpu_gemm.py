@@ -276,3 +276,37 @@ def test_planner_paths_match_the_oracle(amd, M, N, K, expect):
     L = lut32("MBM", 7)
     want = cpu.gemm(L, 7, A[rows].copy(), B)
     assert_close_sum_abs(got[rows], want, cpu.gemm_abs(L, 7, A[rows].copy(), B), 1e-5)
+
+
+def test_gemm_one_term_reductions_cover_every_operand_pattern_width7(amd):
+    """K = 1 makes every output a single product that went through the GEMM kernel's own product
+    form (LUT byte + exponent bits as one FMA factor on the fast path, the full-domain product in
+    flagged chunks): all 2^16 x 2^16 pairs of (sign, exponent, 7-bit mantissa) operand patterns
+    must equal 0 + the oracle's LUT product, bit for bit (NaNs as a class)."""
+    from concurrent.futures import ThreadPoolExecutor
+    from approxtrain_amd import ApproxMulLut
+    from tests.util import lut_bytes, same_bits_or_both_nan
+    _set_split(0)
+    lut = ApproxMulLut(lut_path("MBM", 7))
+    L = cpu.expand_u8(lut_bytes("MBM", 7), 7)
+    n, block = 1 << 16, 1 << 11
+    pats = (np.arange(n, dtype=np.uint32) << 16)
+    A = torch.from_numpy(pats.view(np.float32).reshape(n, 1).copy()).cuda()
+    workers = min(16, cpu.max_threads())
+    a_host = pats.view(np.float32)
+    bad = total = 0
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        for j0 in range(0, n, block):
+            b_host = pats[j0:j0 + block].view(np.float32)
+            got = host(amd.gemm(lut, A, torch.from_numpy(b_host.reshape(1, block).copy()).cuda()))   # [n, block]
+
+            def rows(r):
+                a = np.repeat(a_host[r[0]:r[-1] + 1], block)
+                b = np.tile(b_host, r.size)
+                with np.errstate(invalid="ignore"):
+                    want = cpu.lut_mul_array(L, 7, a, b) + np.float32(0.0)  # the accumulator starts at +0
+                return int((~same_bits_or_both_nan(got[r[0]:r[-1] + 1].ravel(), want)).sum())
+
+            bad += sum(pool.map(rows, np.array_split(np.arange(n), workers * 2)))
+            total += n * block
+    assert total == 1 << 32 and bad == 0, f"{bad} of {total} one-term outputs differ"

@@ -56,3 +56,50 @@ def test_product_m11_legacy_entries():
     got = functors.mul(lut, torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()).cpu().numpy()
     want = cpu.lut_mul_array(img, m, a, b)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def _exhaustive_sweep(kind, m, bits, block):
+    """GPU product (amsim_mul_f32) against the oracle's LUT product over ALL pairs of the 2^bits
+    (sign, exponent, m-bit mantissa) operand patterns, low fraction bits zero: the design of the
+    reference's own sweep (lut/test.cc:41-107), without its exclusion of zero-exponent operands.
+    Operands are generated on the device, block by block; the oracle runs on host threads."""
+    from concurrent.futures import ThreadPoolExecutor
+    from approxtrain_amd import ApproxMulLut, functors
+    lut = ApproxMulLut(lut_path(kind, m))
+    lut32 = cpu.expand_u8(lut_bytes(kind, m), m)
+    shift = 32 - bits
+    n = 1 << bits
+    j_dev = (torch.arange(n, dtype=torch.int64, device="cuda") << shift).to(torch.int32)  # wraps into the sign bit
+    workers = min(16, cpu.max_threads())
+    total = bad = 0
+
+    def oracle(args):
+        a, b = args
+        return cpu.lut_mul_array(lut32, m, a, b)
+
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        for i0 in range(0, n, block):
+            i_dev = (torch.arange(i0, i0 + block, dtype=torch.int64, device="cuda") << shift).to(torch.int32)
+            a_dev = i_dev.repeat_interleave(n).view(torch.float32)
+            b_dev = j_dev.repeat(block).view(torch.float32)
+            got = functors.mul(lut, a_dev, b_dev).cpu().numpy()
+            a, b = a_dev.cpu().numpy(), b_dev.cpu().numpy()
+            parts = np.array_split(np.arange(a.size), workers)
+            want = np.concatenate(list(pool.map(oracle, [(a[p[0]:p[-1] + 1], b[p[0]:p[-1] + 1]) for p in parts])))
+            bad += int((~same_bits_or_both_nan(got, want)).sum())
+            total += a.size
+    assert total == 1 << (2 * bits)
+    assert bad == 0, f"{kind}_{m}: {bad} of {total} products differ from the oracle"
+
+
+@pytest.mark.parametrize("kind", ["MBM", "MIT"])
+def test_exhaustive_top_bit_patterns_width5(kind):
+    """All 2^14 x 2^14 = 2^28 pairs of (sign, exponent, 5-bit mantissa) patterns."""
+    _exhaustive_sweep(kind, 5, 14, 1 << 10)
+
+
+@pytest.mark.parametrize("kind", ["MBM", "MIT"])
+def test_exhaustive_top_bit_patterns_width7(kind):
+    """All 2^16 x 2^16 = 2^32 pairs of (sign, exponent, 7-bit mantissa) patterns: every operand
+    the truncating multiplier can tell apart, crossed with every other one."""
+    _exhaustive_sweep(kind, 7, 16, 1 << 10)
