@@ -63,6 +63,7 @@ SIGNATURES = {
     "amsim_attention_grad_f32": (_i, [_p, _f, _f, _f, _f, _f] + [_i] * 5 + [C.c_float, _f, _f, _f, _p, _sz, _p]),
     "amsim_conv_geometry": (_i, [_i, _i, _i, _i, C.POINTER(_i), C.POINTER(_i)]),
     "amsim_set_split_k": (_i, [_i]),
+    "amsim_set_engine": (_i, [_i]),
     "amsim_calibration_copy": (_i, [_f, _f, _sz, _p]),
     "amsim_microbench_wide": (_i, [_i, _i, _i, _i, _p, _p, _sz, _f, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "amsim_microbench": (_i, [_i, _i, _i, _i, _p, _f, C.POINTER(C.c_double), C.POINTER(C.c_double)]),

@@ -9,6 +9,7 @@
 
 namespace amsim {
 void set_split_k(int mode);
+void set_engine(int mode);
 }
 
 using namespace amsim;
@@ -114,6 +115,14 @@ extern "C" {
 int amsim_set_split_k(int mode)
 {
     amsim::set_split_k(mode);
+    return AMSIM_OK;
+}
+
+int amsim_set_engine(int mode)
+{
+    if (mode != AMSIM_ENGINE_AUTO && mode != AMSIM_ENGINE_LDS_TABLE && mode != AMSIM_ENGINE_DIRECT)
+        return fail(AMSIM_ERR_INVALID, "unknown engine mode");
+    amsim::set_engine(mode);
     return AMSIM_OK;
 }
 

@@ -41,6 +41,7 @@
 namespace amsim {
 
 static std::atomic<int> g_split_k{1};
+static std::atomic<int> g_engine{AMSIM_ENGINE_AUTO};
 
 // staging modes of the lane operand
 enum { STAGE_R = 0,   // threads run along r, one element each (source contiguous in r)
@@ -626,16 +627,6 @@ void lutgemm_kernel(KArgs a)
     }
 }
 
-// sums the split partials in ascending split order (deterministic)
-struct RArgs {
-    const float *partial;
-    float *out;
-    int64_t R, J, Rp, so_r, so_j, out_batch_stride;  // R rows starting at row_base
-    int Jp, nsplit, batch;
-    int64_t row_base;
-    Epilogue ep;
-};
-
 // OUTS consecutive outputs per workgroup, WG_THREADS / OUTS threads ("ways") per output.  Each
 // way takes every ways-th split in eight interleaved chains (eight loads in flight); the chains
 // and then the ways' sums are combined in a fixed order, so the result does not depend on
@@ -729,7 +720,7 @@ int launch_skipped_tap_poison(const float *filter, int KH, int KW, int IC, int O
     return AMSIM_OK;
 }
 
-static void launch_reduce(const RArgs &ra, hipStream_t stream)
+void launch_reduce(const RArgs &ra, hipStream_t stream)
 {
     const int64_t outs = ra.R * ra.J;
     if (outs * ra.batch <= 16384 && ra.nsplit >= 64)
@@ -904,6 +895,7 @@ size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
     size_t need = make_plan(R, J, K, batch, q_batches, false, WAVES_PER_SIMD).total;
     for (int w = WAVES_PER_SIMD - 1; w <= WAVES_PER_SIMD; ++w)
         need = std::max(need, make_plan(R, J, K, batch, q_batches, true, w).total);
+    if (direct_shape_eligible(R, J, K, batch, true)) need = std::max(need, direct_workspace_bytes(R, J, K, batch));
     return need;
 }
 
@@ -1001,6 +993,19 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     }
     if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
+    const int engine = g_engine.load();
+    const bool use_direct = engine != AMSIM_ENGINE_LDS_TABLE && direct_eligible(lut.m, d, engine == AMSIM_ENGINE_DIRECT);
+    // the handle's own setting wins over the process default (read once per call)
+    const bool may_split = (lut.split_k >= 0 ? lut.split_k != 0 : g_split_k.load() != 0) && !d.no_split;
+    // The workspace must be what the query returns (valid for every engine and split mode), whichever
+    // engine runs; a call that keeps its reduction whole on purpose needs only its own plan's share.
+    const size_t need = !d.no_split ? gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches)
+                        : use_direct ? 0
+                                     : make_plan(d.R, d.J, d.K, d.batch, d.q.batches, false, waves64_of(d.p, d.K)).total;
+    if (need && (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need))
+        return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
+                                             std::to_string(need) + " bytes");
+    if (use_direct) return run_gemm_direct(lut, d, may_split, workspace, workspace_bytes, stream);
     if (wide_eligible(lut.m, d)) {
         // tables too wide for the LDS: the row-staged engine, if the workspace also holds the
         // transposed lane operand (else the global-gather variant below does the job, slowly)
@@ -1018,14 +1023,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
             return run_gemm_wide(lut, d, WideQ{qa.qw, qa.qflags, qa.qdesc_out, pq.Jp, pq.nchunks}, ws + pq.total, stream);
         }
     }
-    // the handle's own setting wins over the process default (read once per call)
-    const bool may_split = (lut.split_k >= 0 ? lut.split_k != 0 : g_split_k.load() != 0) && !d.no_split;
     const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, may_split, waves64_of(d.p, d.K));
-    // the size the query returns (valid for either split mode), not just this plan's
-    const size_t need = d.no_split ? pl.total : gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
-    if (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need)
-        return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
-                                             std::to_string(need) + " bytes");
     uint8_t *ws = static_cast<uint8_t *>(workspace);
 
     QArgs qa{};
@@ -1121,5 +1119,6 @@ int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_
 }
 
 void set_split_k(int mode) { g_split_k.store(mode ? 1 : 0); }
+void set_engine(int mode) { g_engine.store(mode); }
 
 }  // namespace amsim

@@ -73,6 +73,18 @@ __device__ __forceinline__ uint32_t q_raw_bits(const QD &q, const float *base, u
 }
 
 
+// sums the split partials in ascending split order (deterministic)
+struct RArgs {
+    const float *partial;
+    float *out;
+    int64_t R, J, Rp, so_r, so_j, out_batch_stride;  // R rows starting at row_base
+    int Jp, nsplit, batch;
+    int64_t row_base;
+    Epilogue ep;
+};
+
+void launch_reduce(const RArgs &ra, hipStream_t stream);
+
 // Decodes the uniform operand into the workspace (qw, qflags) and leaves a copy of its
 // descriptor in device memory (defined with the LDS-table engine).
 int launch_q_prepass(const QArgs &qa, int q_batches, hipStream_t stream);

@@ -138,6 +138,16 @@ int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_
 // what the row-staged engine needs
 size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
 
+// ---- the direct engine for small problems (one launch, operands read where they lie) ----------
+// Tables that fit the LDS only; which problems it takes is decided in direct_eligible().
+constexpr double DIRECT_MAX_MACS = 48.0e6;
+constexpr double DIRECT_MAX_MACS_FEW_OUTPUTS = 160.0e6;
+constexpr double DIRECT_MAX_MACS_ANY = 1.0e10;
+bool direct_shape_eligible(int64_t R, int64_t J, int64_t K, int batch, bool any_size);
+bool direct_eligible(int m, const GemmDesc &d, bool any_size);
+size_t direct_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch);
+int run_gemm_direct(const Lut &lut, const GemmDesc &d, bool may_split, void *workspace, size_t workspace_bytes, hipStream_t stream);
+
 int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream);
 
 // Strided grad-input runs one sub-problem per residue class of the input pixels, each over the

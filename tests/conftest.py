@@ -15,3 +15,18 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def golden_dir():
     return os.path.join(ROOT, "tests", "golden")
+
+
+ENGINES = {"auto": 0, "lds_table": 1, "direct": 2}
+
+
+@pytest.fixture(params=list(ENGINES))
+def amsim_engine(request):
+    """Runs a GPU parity test once per GEMM engine setting (amsim_set_engine): picked per problem,
+    LDS-table engine only, direct engine wherever it can index the problem.  Modules opt in with
+    ``pytest.mark.usefixtures("amsim_engine")``."""
+    import approxtrain_amd
+    lib = approxtrain_amd.load_library()
+    assert lib.amsim_set_engine(ENGINES[request.param]) == 0
+    yield request.param
+    lib.amsim_set_engine(0)

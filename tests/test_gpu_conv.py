@@ -8,7 +8,7 @@ from oracle import cpu
 from tests.gpu_util import assert_close_sum_abs, asym_lut_u8, dev, host, lut32
 from tests.util import REF_CONV_SHAPES, lut_path, small_ints, torch_conv_reference
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("amsim_engine")]
 
 
 @pytest.fixture(scope="module")

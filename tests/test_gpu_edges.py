@@ -11,7 +11,7 @@ from oracle import cpu
 from tests.gpu_util import dev, host, lut32
 from tests.util import lut_path
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("amsim_engine")]
 
 
 @pytest.fixture(autouse=True)

@@ -12,7 +12,7 @@ from oracle import cpu
 from tests.gpu_util import assert_close_sum_abs, asym_lut_u8, dev, host, lut32
 from tests.util import lut_path, small_ints
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("amsim_engine")]
 
 
 @pytest.fixture(scope="module")

@@ -12,7 +12,7 @@ from oracle import cpu
 from tests.gpu_util import assert_close_sum_abs, dev, host, lut32
 from tests.util import lut_path, same_bits_or_both_nan
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("amsim_engine")]
 
 
 SPECIALS = np.array([np.inf, -np.inf, np.nan, 1e-40, -1e-42, 3e38, -3e38, 1e-30, 2e-38, 0.0, -0.0], dtype=np.float32)

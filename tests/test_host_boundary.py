@@ -93,7 +93,7 @@ def test_no_entry_point_crashes_on_null_or_odd_arguments():
     lib = approxtrain_amd.load_library()
     other = {"amsim_status_string", "amsim_last_error", "amsim_device_info", "amsim_lut_load_file", "amsim_lut_create",
              "amsim_lut_destroy", "amsim_lut_mant_width", "amsim_lut_params", "amsim_lut_generate",
-             "amsim_lut_generate_builtin", "amsim_microbench", "amsim_calibration_copy", "amsim_set_split_k",
+             "amsim_lut_generate_builtin", "amsim_microbench", "amsim_calibration_copy", "amsim_set_split_k", "amsim_set_engine",
              "amsim_conv_geometry", "amsim_gemm_plan_info"}
     for name, (res, args) in _lib.SIGNATURES.items():
         if name in other:
