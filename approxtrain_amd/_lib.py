@@ -34,6 +34,7 @@ SIGNATURES = {
     "amsim_lut_mant_width": (_i, [_p]),
     "amsim_lut_params": (_i, [_p, C.POINTER(C.c_uint32), C.POINTER(_i), C.POINTER(_i)]),
     "amsim_lut_set_split_k": (_i, [_p, _i]),
+    "amsim_lut_set_engine": (_i, [_p, _i]),
     "amsim_lut_generate": (_i, [_p, _p, _i, _i, _p, _sz]),
     "amsim_lut_generate_builtin": (_i, [C.c_char_p, _i, _i, _p, _sz]),
     "amsim_mul_f32": (_i, [_p, _f, _f, _f, _sz, _p]),

@@ -993,7 +993,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     }
     if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
         return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
-    const int engine = g_engine.load();
+    const int engine = lut.engine >= 0 ? lut.engine : g_engine.load();  // the handle's own setting wins
     const bool use_direct = engine != AMSIM_ENGINE_LDS_TABLE && direct_eligible(lut.m, d, engine == AMSIM_ENGINE_DIRECT);
     // the handle's own setting wins over the process default (read once per call)
     const bool may_split = (lut.split_k >= 0 ? lut.split_k != 0 : g_split_k.load() != 0) && !d.no_split;

@@ -33,6 +33,7 @@ struct Lut {
     int m = 0;
     int device = 0;
     int split_k = -1;  // how reductions may be run for calls through this handle: -1 process default, 0 whole, 1 split
+    int engine = -1;   // which GEMM engine serves calls through this handle: -1 process default, else AMSIM_ENGINE_*
     size_t entries = 0;
     uint8_t *img_ab = nullptr;
     uint8_t *img_ba = nullptr;

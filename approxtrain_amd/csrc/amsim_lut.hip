@@ -243,6 +243,14 @@ int amsim_lut_destroy(amsim_lut_t lut)
 
 int amsim_lut_mant_width(amsim_lut_t lut) { return lut ? lut->l.m : -1; }
 
+int amsim_lut_set_engine(amsim_lut_t lut, int mode)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (mode < -1 || mode > AMSIM_ENGINE_DIRECT) return fail(AMSIM_ERR_INVALID, "engine mode must be -1 (process default) or an AMSIM_ENGINE_* value");
+    lut->l.engine = mode;
+    return AMSIM_OK;
+}
+
 int amsim_lut_set_split_k(amsim_lut_t lut, int mode)
 {
     if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");

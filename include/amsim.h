@@ -254,7 +254,7 @@ int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, i
  * amsim_set_split_k sets the process default that handles in mode -1 follow (see
  * amsim_lut_set_split_k for the two modes and their tolerance); the initial default is 1. */
 int amsim_set_split_k(int mode);
-/* Which GEMM engine serves tables that fit the LDS (process-wide; for tests and tuning):
+/* Which GEMM engine serves tables that fit the LDS (process-wide default; for tests and tuning):
  * AUTO picks per problem -- the direct engine (one launch, operands read where they lie, built
  * for latency) for small problems, the LDS-table engine (operand pre-pass, LDS-staged tiles, built
  * for throughput) for the rest; LDS_TABLE never uses the direct engine; DIRECT uses it for
@@ -264,6 +264,9 @@ int amsim_set_split_k(int mode);
 #define AMSIM_ENGINE_LDS_TABLE 1
 #define AMSIM_ENGINE_DIRECT 2
 int amsim_set_engine(int mode);
+/* The same choice for calls through one handle (-1, the initial value, follows the process-wide
+ * setting): lets threads hold different settings without sharing mutable state. */
+int amsim_lut_set_engine(amsim_lut_t lut, int mode);
 /* How a GEMM of this shape would be run when reductions may be split (contiguous, aligned
  * operands assumed): info = {outputs per lane, row tiles per workgroup, splits of the main part's
  * reduction, chunks (of 32) per split, rows in the main part, splits of the tail rows' reduction

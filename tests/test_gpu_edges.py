@@ -238,3 +238,23 @@ def test_library_loaded_before_torch_still_shares_its_runtime():
     run = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stderr[-2000:]
     assert "sum 512.0" in run.stdout
+
+
+def test_per_handle_engine_and_reduction_settings_override_the_process_defaults():
+    """Two handles of one table with different settings in one process: each call follows its own
+    handle (amsim_lut_set_engine / amsim_lut_set_split_k), whatever the process-wide defaults say."""
+    import approxtrain_amd
+    from approxtrain_amd import ApproxMulLut, functors
+    lib = approxtrain_amd.load_library()
+    a, b = ApproxMulLut(lut_path("MBM", 7)), ApproxMulLut(lut_path("MBM", 7))
+    assert lib.amsim_lut_set_engine(a.handle, 1) == 0 and lib.amsim_lut_set_split_k(a.handle, 0) == 0   # LDS-table engine, whole reductions
+    assert lib.amsim_lut_set_engine(b.handle, 2) == 0 and lib.amsim_lut_set_split_k(b.handle, 0) == 0   # direct engine, whole reductions
+    assert lib.amsim_lut_set_engine(a.handle, 3) == 1 and lib.amsim_lut_set_split_k(a.handle, 2) == 1   # refused values
+    rng = np.random.default_rng(21)
+    A = rng.standard_normal((70, 4000)).astype(np.float32)
+    B = rng.standard_normal((4000, 20)).astype(np.float32)
+    want = cpu.gemm(lut32("MBM", 7), 7, A, B)
+    lib.amsim_set_split_k(1)  # the default would split this long reduction over workgroups
+    for lut in (a, b):
+        got = host(functors.gemm(lut, dev(A), dev(B)))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
