@@ -195,7 +195,8 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     // row tile)?  Almost never: then the whole reduction runs the loop nest that holds nothing but
     // fast stages, whose registers the rare path's state cannot crowd.
     int tile_flagged = 0;
-    for (int ch = 0; ch < a.nchunks; ++ch) tile_flagged |= (int)qfl[ch];
+    for (int ch = tid; ch < a.nchunks; ch += WIDE_THREADS)
+        tile_flagged |= (int)a.qflags[(size_t)(by / STRIPS_PER_TILE) * a.nchunks + ch];
     for (int i = tid; i < a.nchunks * (WIDE_TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
         tile_flagged |= (int)a.pflags[(size_t)(i / (WIDE_TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (WIDE_TILE_ROWS / PT_ROWS) +
                                      i % (WIDE_TILE_ROWS / PT_ROWS)];
