@@ -99,8 +99,12 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
     const size_t Kp = (size_t)a.nchunks * KC;
     const size_t tile = ((size_t)qb * ntiles + jt) * Kp * QT + (size_t)ch * KC * QT;
     uint32_t *qw = a.qw + tile;
-    // lanes follow the source's contiguous direction
+    // Lanes follow the source's contiguous direction when reading.  A source that is contiguous
+    // along k would then be written with a 64-byte stride between lanes: its decoded words take a
+    // turn through LDS instead, so that every store covers consecutive words of the tile.
     const bool k_fast = (a.q.kind == Q_DENSE && a.q.sk == 1 && a.q.sj != 1) || (a.q.kind == Q_FLIP);
+    __shared__ uint32_t turn[WG_THREADS / 64][KC][QT + 1];
+    const int w = threadIdx.x >> 6;
     int unsafe = 0;
 #pragma unroll
     for (int i = 0; i < KC * QT / 64; ++i) {
@@ -113,7 +117,17 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
         // zero (and padding) elements select the all-zero LUT row that follows the table:
         // their product term is then exactly +-0 without a test in the inner loop
         const uint32_t mant = (raw & 0x7fffffffu) ? ((raw & 0x7fffffu) >> (23 - a.m)) : (1u << a.m);
-        qw[kk * QT + jj] = (raw & 0xff800000u) | (mant << a.m);
+        const uint32_t word = (raw & 0xff800000u) | (mant << a.m);
+        if (k_fast) turn[w][kk][jj] = word;
+        else qw[e] = word;  // e == kk * QT + jj
+    }
+    if (k_fast) {
+        // (the wavefront reads back what it wrote itself: LDS operations of one wavefront stay in order)
+#pragma unroll
+        for (int i = 0; i < KC * QT / 64; ++i) {
+            const int e = lane + 64 * i;
+            qw[e] = turn[w][e / QT][e % QT];
+        }
     }
     const int any = __any(unsafe);
     if (lane == 0) a.qflags[((size_t)qb * ntiles + jt) * a.nchunks + ch] = (uint32_t)any;
