@@ -43,11 +43,13 @@ SIGNATURES = {
     "amsim_gemm_f32": (_i, [_p, _i, _i, _i, _i64, _i64, _i64, _f, _i64, _f, _i64, _f, _i64,
                             _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "amsim_convam_workspace_bytes": (_sz, [_i] * 7),
+    "amsim_convam_workspace_bytes_for": (_sz, [_p] + [_i] * 7),
     "amsim_convam_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p, _sz, _p]),
     "amsim_convam_noalloc_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p]),
     "amsim_convam_bias_act_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _f, _i, _p, _sz, _p]),
     "amsim_convam_input_grad_workspace_bytes": (_sz, [_i] * 7),
     "amsim_convam_input_grad_strided_workspace_bytes": (_sz, [_i] * 11),
+    "amsim_convam_input_grad_workspace_bytes_for": (_sz, [_p] + [_i] * 11),
     "amsim_convam_input_grad_f32": (_i, [_p, _f, _i, _i, _i, _i, _f] + [_i] * 9 + [_f, _i, _i, _p, _sz, _p]),
     "amsim_convam_filter_grad_workspace_bytes": (_sz, [_i] * 7),
     "amsim_convam_filter_grad_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p, _sz, _p]),

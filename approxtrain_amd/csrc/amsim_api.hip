@@ -168,6 +168,16 @@ size_t amsim_convam_workspace_bytes(int batch, int out_rows, int out_cols, int o
                                 (int64_t)filter_rows * filter_cols * in_depth, 1, 1);
 }
 
+size_t amsim_convam_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols, int out_depth,
+                                        int filter_rows, int filter_cols, int in_depth)
+{
+    size_t need = amsim_convam_workspace_bytes(batch, out_rows, out_cols, out_depth, filter_rows, filter_cols, in_depth);
+    if (need && lut != nullptr && lut->l.m > 7)  // + the im2col the row-staged engine gathers from
+        need = std::max(need, gemm_workspace_bytes_wide((int64_t)batch * out_rows * out_cols, out_depth,
+                                                        (int64_t)filter_rows * filter_cols * in_depth, 1, 1));
+    return need;
+}
+
 int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
                      int out_cols, int out_depth, int stride_cols, int stride_rows, int filter_left_offset,
                      int filter_top_offset, int filter_rows, int filter_cols, int in_depth, int input_cols,
@@ -345,6 +355,25 @@ size_t amsim_convam_input_grad_strided_workspace_bytes(int batch, int input_rows
         for (int px = 0; px < stride_cols; ++px) {
             const GemmDesc d = grad_input_phase(g, py, px, nullptr, nullptr, nullptr);
             need = std::max(need, poison_bytes(in_depth) + gemm_workspace_bytes(d.R, d.J, d.K, 1, 1));
+        }
+    return need;
+}
+
+size_t amsim_convam_input_grad_workspace_bytes_for(amsim_lut_t lut, int batch, int input_rows, int input_cols,
+                                                   int in_depth, int filter_rows, int filter_cols, int out_depth,
+                                                   int stride_rows, int stride_cols, int pad_top, int pad_left)
+{
+    size_t need = amsim_convam_input_grad_strided_workspace_bytes(batch, input_rows, input_cols, in_depth, filter_rows,
+                                                                  filter_cols, out_depth, stride_rows, stride_cols, pad_top,
+                                                                  pad_left);
+    if (!need || lut == nullptr || lut->l.m <= 7 || stride_rows < 1 || stride_cols < 1) return need;
+    const GradInputGeometry g{batch, input_rows, input_cols, in_depth, filter_rows, filter_cols, out_depth,
+                              0, 0, stride_rows, stride_cols, pad_top, pad_left};
+    for (int py = 0; py < stride_rows; ++py)
+        for (int px = 0; px < stride_cols; ++px) {
+            const GemmDesc d = grad_input_phase(g, py, px, nullptr, nullptr, nullptr);
+            const size_t wide = gemm_workspace_bytes_wide(d.R, d.J, d.K, 1, 1);
+            if (wide) need = std::max(need, poison_bytes(in_depth) + wide);
         }
     return need;
 }

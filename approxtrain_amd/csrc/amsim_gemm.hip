@@ -919,12 +919,16 @@ static size_t unsplit_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
     return make_plan(R, J, K, batch, q_batches, false, WAVES_PER_SIMD).total;
 }
 
+size_t gemm_workspace_bytes_wide(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
+{
+    if (R <= 0 || J <= 0 || K <= 0 || batch <= 0 || !wide_shape_eligible(R, batch)) return 0;
+    return unsplit_bytes(R, J, K, batch, q_batches) + wide_workspace_bytes(R, K, batch);
+}
+
 size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 {
-    size_t need = gemm_workspace_bytes(R, J, K, batch, q_batches);
-    if (need && wide_shape_eligible(R, batch))
-        need = std::max(need, unsplit_bytes(R, J, K, batch, q_batches) + wide_workspace_bytes(R, K));
-    return need;
+    const size_t need = gemm_workspace_bytes(R, J, K, batch, q_batches);
+    return need ? std::max(need, gemm_workspace_bytes_wide(R, J, K, batch, q_batches)) : 0;
 }
 
 // what the planner decides for a problem: {TN, WR, nsplit, chunks per split, rows of the main
@@ -1025,7 +1029,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         // transposed lane operand (else the global-gather variant below does the job, slowly)
         const Plan pq = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, false, WAVES_PER_SIMD);
         if (workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-            workspace_bytes >= pq.total + wide_workspace_bytes(d.R, d.K)) {
+            workspace_bytes >= pq.total + wide_workspace_bytes(d.R, d.K, d.batch)) {
             uint8_t *ws = static_cast<uint8_t *>(workspace);
             QArgs qa{};
             qa.q = d.q;

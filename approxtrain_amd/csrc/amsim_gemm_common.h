@@ -85,6 +85,27 @@ struct RArgs {
 
 void launch_reduce(const RArgs &ra, hipStream_t stream);
 
+// raw bits of lane-operand element (r, k) of batch item `base`, whatever the source addressing
+// (dense; im2col-style patch, cuda/cuda_kernel.cu:35-60; filter-gradient gather, :327-353);
+// zero outside R x K and outside the image.  Element by element with divisions: for passes that
+// touch every element once, not for inner loops.
+__device__ __forceinline__ uint32_t p_raw_bits(const PDesc &p, const float *base, int64_t R, int64_t K, int64_t r, int64_t k)
+{
+    if (r >= R || k >= K) return 0u;
+    if (p.kind == P_DENSE) return f2u(base[r * p.sr + k * p.sk]);
+    int b, y, x, fy, fx, c;
+    if (p.kind == P_PATCH) {
+        x = (int)(r % p.GW); const int64_t t = r / p.GW; y = (int)(t % p.GH); b = (int)(t / p.GH);
+        c = (int)(k % p.C); const int u = (int)(k / p.C); fx = u % p.KW; fy = u / p.KW;
+    } else {
+        c = (int)(r % p.C); const int u = (int)(r / p.C); fx = u % p.KW; fy = u / p.KW;
+        x = (int)(k % p.GW); const int64_t t = k / p.GW; y = (int)(t % p.GH); b = (int)(t / p.GH);
+    }
+    const int iy = y * p.sy - p.pt + fy, ix = x * p.sx - p.pl + fx;
+    if ((unsigned)iy >= (unsigned)p.SH || (unsigned)ix >= (unsigned)p.SW) return 0u;
+    return f2u(base[(((int64_t)b * p.SH + iy) * p.SW + ix) * p.C + c]);
+}
+
 // Decodes the uniform operand into the workspace (qw, qflags) and leaves a copy of its
 // descriptor in device memory (defined with the LDS-table engine).
 int launch_q_prepass(const QArgs &qa, int q_batches, hipStream_t stream);

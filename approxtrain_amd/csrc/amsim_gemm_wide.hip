@@ -35,7 +35,7 @@ namespace {
 // A workgroup is 512 threads = 8 wavefronts (one per staged table row) on 4096 rows x 8 columns, and
 // two of them share a compute unit: while one waits at its stage barrier the other gathers (measured
 // 4.7 TMAC/s against 4.45 for one 1024-thread workgroup on 16 columns).
-constexpr int WIDE_TILE_ROWS = 4096;              // rows per workgroup
+constexpr int WIDE_TILE_ROWS = 4096;              // rows per workgroup (half of that when workgroups are too few, below)
 constexpr int WIDE_TN = 8;                        // columns per workgroup: half a tile of the pre-decoded operand
 constexpr int WIDE_THREADS = WIDE_TN * 64;
 constexpr int WIDE_SLOT_BYTES = 4096;             // LDS bytes reserved per staged table row (2^11 entries x 2)
@@ -45,20 +45,26 @@ struct PTArgs {
     PDesc p;
     int64_t R, K, Rp;
     int nchunks;
-    uint32_t *pt;      // [nchunks * KC][Rp] raw bits
-    uint32_t *pflags;  // [nchunks][Rp / 64]
+    uint32_t *pt;      // [batch][nchunks * KC][Rp] raw bits
+    uint32_t *pflags;  // [batch][nchunks][Rp / 64]
 };
 
-// One workgroup per (64-row group, 32-deep chunk): reads the tile along the source's contiguous
-// direction, writes it in [k][row] order, flags it if it holds an operand the fast product path
-// cannot take.
+// One workgroup per (64-row group, 32-deep chunk) and batch item (blockIdx.y): reads the tile along
+// the source's contiguous direction -- for patch sources this IS the im2col the reference
+// materialises (cuda/cuda_kernel.cu:35-60), here transposed -- writes it in [k][row] order, flags it
+// if it holds an operand the fast product path cannot take.
 __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
 {
     __shared__ uint32_t tile[KC][PT_ROWS + 1];
     const int64_t G = a.Rp / PT_ROWS;
     const int64_t g = blockIdx.x % G, ch = blockIdx.x / G;
+    const int bz = blockIdx.y;
     const int tid = threadIdx.x;
-    const bool k_fast = a.p.sk == 1 && a.p.sr != 1;
+    const float *pbase = a.p.base + (int64_t)bz * a.p.batch_stride;
+    uint32_t *pt = a.pt + (size_t)bz * a.nchunks * KC * a.Rp;
+    // lanes along k where the source is contiguous there: row-major dense operands, and patches
+    // (channels run fastest in both the image and the reduction index)
+    const bool k_fast = a.p.kind == P_PATCH || (a.p.kind == P_DENSE && a.p.sk == 1 && a.p.sr != 1);
     int unsafe = 0;
 #pragma unroll
     for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
@@ -67,8 +73,7 @@ __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
         if (k_fast) { kk = e % KC; rl = e / KC; }
         else { rl = e % PT_ROWS; kk = e / PT_ROWS; }
         const int64_t r = g * PT_ROWS + rl, k = ch * KC + kk;
-        uint32_t raw = 0;
-        if (r < a.R && k < a.K) raw = f2u(a.p.base[r * a.p.sr + k * a.p.sk]);
+        const uint32_t raw = p_raw_bits(a.p, pbase, a.R, a.K, r, k);
         unsafe |= operand_unsafe(raw) ? 1 : 0;
         tile[kk][rl] = raw;
     }
@@ -77,9 +82,9 @@ __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
     for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
         const int e = tid + WG_THREADS * i;
         const int rl = e % PT_ROWS, kk = e / PT_ROWS;
-        a.pt[(size_t)(ch * KC + kk) * a.Rp + g * PT_ROWS + rl] = tile[kk][rl];
+        pt[(size_t)(ch * KC + kk) * a.Rp + g * PT_ROWS + rl] = tile[kk][rl];
     }
-    if (tid == 0) a.pflags[ch * G + g] = (uint32_t)any;
+    if (tid == 0) a.pflags[((size_t)bz * a.nchunks + ch) * G + g] = (uint32_t)any;
 }
 
 // LDS byte address of a pointer into a __shared__ object
@@ -121,18 +126,21 @@ struct WArgs {
     int64_t R, J, K, Rp;
     int Jp, nchunks;
     float *out;
-    int64_t so_r, so_j;
+    int64_t so_r, so_j, out_batch_stride;
     int vec_store;
+    int q_batches;           // 1: the uniform operand is shared by every batch item
     Epilogue ep;
-    unsigned X, Y;           // row tiles, column strips
+    unsigned X, Y;           // row tiles, column strips (blockIdx.y runs over the batch)
 };
 
 // PARTS: KB of a table row copied per stage and slot (4 at width 11, 2 at width 10, 1 below: the copy
 // of a narrower row runs on into the rows behind it, which the image's padding keeps in bounds).
-template <int PARTS>
+// RPT: rows per thread, 8 (4096 rows per workgroup: 1 byte of table row pulled per product) or 4 (2048
+// rows, 2 bytes per product: for problems that would otherwise leave compute units without a workgroup).
+template <int PARTS, int RPT>
 __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
 {
-    constexpr int WIDE_RPT = WIDE_TILE_ROWS / WIDE_THREADS;
+    constexpr int TILE_ROWS = WIDE_THREADS * RPT;
     constexpr int WIDE_BUF_BYTES = WIDE_TN * WIDE_SLOT_BYTES;
     // Two halves of 8 slots x 4 KB, as two objects: the compiler then knows that the direct-to-LDS
     // copies into one half do not alias the gathers from the other, and does not make the gathers
@@ -152,19 +160,22 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         by = V % a.Y;
         bx = V / a.Y;
     }
-    const int64_t row0 = (int64_t)bx * WIDE_TILE_ROWS;
+    const int64_t row0 = (int64_t)bx * TILE_ROWS;
     const int j0 = by * WIDE_TN;
     constexpr int STRIPS_PER_TILE = QT / WIDE_TN;
     const int m = a.m, mshift = 23 - m;
     const uint32_t mmask = (1u << m) - 1u;
     const int Kp = a.nchunks * KC;
-    const cq1_t qtile = (cq1_t)(uintptr_t)(a.qw + (size_t)(by / STRIPS_PER_TILE) * Kp * QT + (by % STRIPS_PER_TILE) * WIDE_TN);
-    const cq1_t qfl = (cq1_t)(uintptr_t)(a.qflags + (size_t)(by / STRIPS_PER_TILE) * a.nchunks);
-    const uint32_t *pcol = a.pt + row0 + tid;
+    const int bz = blockIdx.y, qb = a.q_batches > 1 ? bz : 0;
+    const size_t qt_index = (size_t)qb * (a.Jp / QT) + by / STRIPS_PER_TILE;  // tile of the pre-decoded operand
+    const cq1_t qtile = (cq1_t)(uintptr_t)(a.qw + qt_index * Kp * QT + (by % STRIPS_PER_TILE) * WIDE_TN);
+    const cq1_t qfl = (cq1_t)(uintptr_t)(a.qflags + qt_index * a.nchunks);
+    const uint32_t *pcol = a.pt + (size_t)bz * Kp * a.Rp + row0 + tid;
     const int64_t G = a.Rp / PT_ROWS;
-    float acc[WIDE_RPT][WIDE_TN];
+    const uint32_t *pfl = a.pflags + (size_t)bz * a.nchunks * G;
+    float acc[RPT][WIDE_TN];
 #pragma unroll
-    for (int rr = 0; rr < WIDE_RPT; ++rr)
+    for (int rr = 0; rr < RPT; ++rr)
 #pragma unroll
         for (int j = 0; j < WIDE_TN; ++j) acc[rr][j] = 0.0f;
 
@@ -180,10 +191,10 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
 #endif
         }
     };
-    uint32_t pc[WIDE_RPT], pn[WIDE_RPT];
-    auto load_p = [&](int k, uint32_t (&dst)[WIDE_RPT]) {
+    uint32_t pc[RPT], pn[RPT];
+    auto load_p = [&](int k, uint32_t (&dst)[RPT]) {
 #pragma unroll
-        for (int rr = 0; rr < WIDE_RPT; ++rr) dst[rr] = pcol[(size_t)k * a.Rp + rr * WIDE_THREADS];
+        for (int rr = 0; rr < RPT; ++rr) dst[rr] = pcol[(size_t)k * a.Rp + rr * WIDE_THREADS];
     };
 
     fill(0, rows_a);
@@ -196,10 +207,10 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     // fast stages, whose registers the rare path's state cannot crowd.
     int tile_flagged = 0;
     for (int ch = tid; ch < a.nchunks; ch += WIDE_THREADS)
-        tile_flagged |= (int)a.qflags[(size_t)(by / STRIPS_PER_TILE) * a.nchunks + ch];
-    for (int i = tid; i < a.nchunks * (WIDE_TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
-        tile_flagged |= (int)a.pflags[(size_t)(i / (WIDE_TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (WIDE_TILE_ROWS / PT_ROWS) +
-                                     i % (WIDE_TILE_ROWS / PT_ROWS)];
+        tile_flagged |= (int)a.qflags[qt_index * a.nchunks + ch];
+    for (int i = tid; i < a.nchunks * (TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
+        tile_flagged |= (int)pfl[(size_t)(i / (TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (TILE_ROWS / PT_ROWS) +
+                                 i % (TILE_ROWS / PT_ROWS)];
     tile_flagged = __syncthreads_or(tile_flagged);
 
     // one stage: copies for stage k + 1 go into `next` while stage k gathers from `cur`
@@ -215,7 +226,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
 #pragma unroll
             for (int j = 0; j < WIDE_TN; ++j) qt[j] = qtile[k * QT + j] & 0xff800000u;
 #pragma unroll
-            for (int rr = 0; rr < WIDE_RPT; ++rr) {
+            for (int rr = 0; rr < RPT; ++rr) {
                 const float ta = u2f(pc[rr] & 0xff800000u);
                 const uint32_t off = ((pc[rr] >> mshift) & mmask) << 1;
                 uint32_t e[WIDE_TN];
@@ -232,16 +243,16 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
             // registers.
             const __attribute__((address_space(4))) QDesc &qd = *(const __attribute__((address_space(4))) QDesc *)(uintptr_t)a.qdesc;
             const float *qsrc = qd.base;
-            float tmp[WIDE_RPT * WIDE_TN];
-            uint32_t praw[WIDE_RPT];
+            float tmp[RPT * WIDE_TN];
+            uint32_t praw[RPT];
 #pragma unroll
-            for (int rr = 0; rr < WIDE_RPT; ++rr) {
+            for (int rr = 0; rr < RPT; ++rr) {
                 praw[rr] = pc[rr];
 #pragma unroll
                 for (int j = 0; j < WIDE_TN; ++j) tmp[rr * WIDE_TN + j] = acc[rr][j];
             }
 #pragma unroll 1
-            for (int idx = 0; idx < WIDE_RPT * WIDE_TN; ++idx) {
+            for (int idx = 0; idx < RPT * WIDE_TN; ++idx) {
                 const int rr = idx / WIDE_TN, j = idx % WIDE_TN;
                 const uint32_t raw = praw[rr];
                 const uint32_t off = ((raw >> mshift) & mmask) << 1;
@@ -250,12 +261,12 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
                 tmp[idx] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
             }
 #pragma unroll
-            for (int rr = 0; rr < WIDE_RPT; ++rr)
+            for (int rr = 0; rr < RPT; ++rr)
 #pragma unroll
                 for (int j = 0; j < WIDE_TN; ++j) acc[rr][j] = tmp[rr * WIDE_TN + j];
         }
 #pragma unroll
-        for (int rr = 0; rr < WIDE_RPT; ++rr) pc[rr] = pn[rr];
+        for (int rr = 0; rr < RPT; ++rr) pc[rr] = pn[rr];
         // my copies for the next stage have landed; after the barrier so have everyone's, and
         // every wavefront is done gathering from this stage's half
         __builtin_amdgcn_sched_barrier(0);
@@ -270,7 +281,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         }
     } else {
         for (int ch = 0; ch < a.nchunks; ++ch) {
-            const uint32_t pf = a.pflags[(size_t)ch * G + (size_t)bx * (WIDE_TILE_ROWS / PT_ROWS) + lane];
+            const uint32_t pf = lane < TILE_ROWS / PT_ROWS ? pfl[(size_t)ch * G + (size_t)bx * (TILE_ROWS / PT_ROWS) + lane] : 0u;
             const bool unsafe = (qfl[ch] != 0u) | (__any(pf != 0u) != 0);
             if (!unsafe) {
 #pragma unroll 1
@@ -289,10 +300,10 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     }
 
 #pragma unroll
-    for (int rr = 0; rr < WIDE_RPT; ++rr) {
+    for (int rr = 0; rr < RPT; ++rr) {
         const int64_t r = row0 + rr * WIDE_THREADS + tid;
         if (r >= a.R) continue;
-        float *o = a.out + out_row_offset(a.ep.omap, r, a.so_r);
+        float *o = a.out + (int64_t)bz * a.out_batch_stride + out_row_offset(a.ep.omap, r, a.so_r);
         if (a.ep.bias_j || a.ep.bias_r || a.ep.act) {
 #pragma unroll
             for (int j = 0; j < WIDE_TN; ++j) acc[rr][j] = apply_epilogue(a.ep, acc[rr][j], r, min((int64_t)(j0 + j), a.J - 1));
@@ -315,17 +326,21 @@ inline int64_t padded_rows(int64_t R) { return (R + WIDE_TILE_ROWS - 1) / WIDE_T
 
 }  // namespace
 
-bool wide_shape_eligible(int64_t R, int batch) { return batch == 1 && R >= WIDE_MIN_ROWS; }
+bool wide_shape_eligible(int64_t R, int batch) { return batch >= 1 && batch <= 65535 && R >= WIDE_MIN_ROWS; }
 
+// Dense and patch (forward / input-gradient convolution) lane operands; the filter gradient's rows
+// are the few filter elements and its reduction the many pixels, the opposite of what this engine
+// needs, so it stays on the global-gather variant.
 bool wide_eligible(int m, const GemmDesc &d)
 {
-    return m > 7 && d.p.kind == P_DENSE && !d.omap.enabled && wide_shape_eligible(d.R, d.batch);
+    return m > 7 && (d.p.kind == P_DENSE || d.p.kind == P_PATCH) && wide_shape_eligible(d.R, d.batch);
 }
 
-size_t wide_workspace_bytes(int64_t R, int64_t K)
+size_t wide_workspace_bytes(int64_t R, int64_t K, int batch)
 {
     const int64_t Rp = padded_rows(R), nchunks = (K + KC - 1) / KC;
-    return align256((size_t)nchunks * KC * Rp * sizeof(uint32_t)) + align256((size_t)nchunks * (Rp / PT_ROWS) * sizeof(uint32_t));
+    return align256((size_t)batch * nchunks * KC * Rp * sizeof(uint32_t)) +
+           align256((size_t)batch * nchunks * (Rp / PT_ROWS) * sizeof(uint32_t));
 }
 
 int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, hipStream_t stream)
@@ -336,10 +351,10 @@ int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_
     PTArgs pa{};
     pa.p = d.p; pa.R = d.R; pa.K = d.K; pa.Rp = Rp; pa.nchunks = q.nchunks;
     pa.pt = reinterpret_cast<uint32_t *>(ws);
-    pa.pflags = reinterpret_cast<uint32_t *>(ws + align256((size_t)q.nchunks * KC * Rp * sizeof(uint32_t)));
+    pa.pflags = reinterpret_cast<uint32_t *>(ws + align256((size_t)d.batch * q.nchunks * KC * Rp * sizeof(uint32_t)));
     const int64_t pwgs = G * q.nchunks;
     if (pwgs >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "lane operand exceeds the grid limit");
-    p_linear_kernel<<<dim3((unsigned)pwgs), WG_THREADS, 0, stream>>>(pa);
+    p_linear_kernel<<<dim3((unsigned)pwgs, (unsigned)d.batch), WG_THREADS, 0, stream>>>(pa);
     AMSIM_HIP_CHECK(hipGetLastError());
 
     WArgs wa{};
@@ -349,16 +364,29 @@ int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_
     wa.m = lut.m; wa.lane_first = d.lane_first ? 1 : 0;
     wa.R = d.R; wa.J = d.J; wa.K = d.K; wa.Rp = Rp;
     wa.Jp = q.Jp; wa.nchunks = q.nchunks;
-    wa.out = d.out; wa.so_r = d.so_r; wa.so_j = d.so_j;
-    wa.vec_store = (d.so_j == 1 && d.so_r % 4 == 0 && ((uintptr_t)d.out & 15) == 0) ? 1 : 0;
+    wa.out = d.out; wa.so_r = d.so_r; wa.so_j = d.so_j; wa.out_batch_stride = d.out_batch_stride;
+    wa.vec_store = (d.so_j == 1 && d.so_r % 4 == 0 && d.out_batch_stride % 4 == 0 && ((uintptr_t)d.out & 15) == 0) ? 1 : 0;
+    wa.q_batches = d.q.batches;
     wa.ep = Epilogue{d.bias_j, d.bias_r, d.act, d.omap};
-    wa.X = (unsigned)(Rp / WIDE_TILE_ROWS);
-    wa.Y = (unsigned)(q.Jp / WIDE_TN);
+    // half-height tiles when full-height ones would leave workgroup slots (two per compute unit) empty
+    const int64_t strips = q.Jp / WIDE_TN;
+    const bool half = (Rp / WIDE_TILE_ROWS) * strips * d.batch < 2 * (int64_t)device_compute_units();
+    const int tile_rows = half ? WIDE_TILE_ROWS / 2 : WIDE_TILE_ROWS;
+    wa.X = (unsigned)((d.R + tile_rows - 1) / tile_rows);
+    wa.Y = (unsigned)strips;
     const int64_t total = (int64_t)wa.X * wa.Y;
     if (total >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "workgroup count exceeds the grid limit");
-    if (lut.m >= 11) lutgemm_wide_kernel<4><<<dim3((unsigned)total), WIDE_THREADS, 0, stream>>>(wa);
-    else if (lut.m == 10) lutgemm_wide_kernel<2><<<dim3((unsigned)total), WIDE_THREADS, 0, stream>>>(wa);
-    else lutgemm_wide_kernel<1><<<dim3((unsigned)total), WIDE_THREADS, 0, stream>>>(wa);
+    const dim3 grid((unsigned)total, (unsigned)d.batch);
+    const int parts = lut.m >= 11 ? 4 : lut.m == 10 ? 2 : 1;
+    if (half) {
+        if (parts == 4) lutgemm_wide_kernel<4, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        else if (parts == 2) lutgemm_wide_kernel<2, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        else lutgemm_wide_kernel<1, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+    } else {
+        if (parts == 4) lutgemm_wide_kernel<4, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        else if (parts == 2) lutgemm_wide_kernel<2, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        else lutgemm_wide_kernel<1, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+    }
     AMSIM_HIP_CHECK(hipGetLastError());
     return AMSIM_OK;
 }

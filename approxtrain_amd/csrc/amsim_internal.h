@@ -121,9 +121,10 @@ void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, b
 int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream);
 
 // ---- the row-staged engine for tables too wide for the LDS (mantissa widths 8..11) ----------
-// Serves dense, unbatched problems with at least WIDE_MIN_ROWS rows when the caller's workspace
-// also holds the transposed lane operand (wide_workspace_bytes on top of the unsplit plan);
-// everything else with such tables runs on the LDS-table engine's global-gather variant.
+// Serves dense and patch (convolution forward / input gradient) problems with at least
+// WIDE_MIN_ROWS rows per batch item when the caller's workspace also holds the transposed lane
+// operand (wide_workspace_bytes on top of the unsplit plan); everything else with such tables
+// runs on the LDS-table engine's global-gather variant.
 constexpr int64_t WIDE_MIN_ROWS = 1024;
 struct WideQ {
     const uint32_t *qw;
@@ -133,11 +134,13 @@ struct WideQ {
 };
 bool wide_shape_eligible(int64_t R, int batch);
 bool wide_eligible(int m, const GemmDesc &d);
-size_t wide_workspace_bytes(int64_t R, int64_t K);
+size_t wide_workspace_bytes(int64_t R, int64_t K, int batch);
 int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, hipStream_t stream);
 // workspace that serves a dense problem with any table: the larger of gemm_workspace_bytes and
 // what the row-staged engine needs
 size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
+// what the row-staged engine needs for a problem in all (unsplit plan + transposed lane operand)
+size_t gemm_workspace_bytes_wide(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
 
 // ---- the direct engine for small problems (one launch, operands read where they lie) ----------
 // Tables that fit the LDS only; which problems it takes is decided in direct_eligible().

@@ -111,7 +111,7 @@ def convam(lut, input, filter, strides=(1, 1), padding="SAME", bias=None, activa
     ow, pl = conv_geometry(wd, kw, strides[1], padding)
     out = torch.empty((n, oh, ow, oc), dtype=torch.float32, device=x.device)
     lib = load_library()
-    nbytes = lib.amsim_convam_workspace_bytes(n, oh, ow, oc, kh, kw, c)
+    nbytes = lib.amsim_convam_workspace_bytes_for(lut.handle, n, oh, ow, oc, kh, kw, c)
     ws, wsp = _workspace(nbytes, x.device)
     if b is None and act == 0:
         check(lib.amsim_convam_f32(lut.handle, _ptr(x), _ptr(out), n, oh, ow, oc, strides[1], strides[0], pl, pt,
@@ -136,8 +136,8 @@ def convam_input_grad(lut, input_sizes, filter, out_backprop, strides=(1, 1), pa
     hole_h = (oh - 1) * strides[0] + 1 if oh > 0 else 0
     hole_w = (ow - 1) * strides[1] + 1 if ow > 0 else 0
     lib = load_library()
-    nbytes = lib.amsim_convam_input_grad_strided_workspace_bytes(n, h, wd, c, kh, kw, oc, strides[0], strides[1],
-                                                                 kh - 1 - pt, kw - 1 - pl)
+    nbytes = lib.amsim_convam_input_grad_workspace_bytes_for(lut.handle, n, h, wd, c, kh, kw, oc, strides[0], strides[1],
+                                                             kh - 1 - pt, kw - 1 - pl)
     ws, wsp = _workspace(nbytes, dy.device)
     check(lib.amsim_convam_input_grad_f32(lut.handle, _ptr(dy), hole_w, hole_h, kh - 1 - pt, kw - 1 - pl, _ptr(w),
                                           kh, kw, oc, strides[0], strides[1], n, h, wd, c, _ptr(out), oh, ow,

@@ -131,6 +131,13 @@ int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_dat
                      int filter_top_offset, int filter_rows, int filter_cols, int in_depth, int input_cols,
                      int input_rows, const float *filter, void *workspace, size_t workspace_bytes,
                      void *stream);
+/* The query for a given table.  For tables of up to 7 mantissa bits it equals the one above.  For
+ * wider tables (8..11 bits) it adds what the row-staged engine needs -- an im2col of the input, the
+ * temporary the reference also allocates (convam.cc:518-546) -- so that the call runs on that engine
+ * (about 10x faster) instead of one global gather per product; a call given only the smaller amount
+ * still runs, on the slow path. */
+size_t amsim_convam_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols, int out_depth,
+                                        int filter_rows, int filter_cols, int in_depth);
 
 /* amsim_convam_f32 for callers that cannot allocate device memory or bring a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
@@ -172,6 +179,10 @@ size_t amsim_convam_input_grad_workspace_bytes(int batch, int input_rows, int in
 size_t amsim_convam_input_grad_strided_workspace_bytes(int batch, int input_rows, int input_cols, int in_depth,
                                                        int filter_rows, int filter_cols, int out_depth,
                                                        int stride_rows, int stride_cols, int pad_top, int pad_left);
+/* The strided query for a given table: as amsim_convam_workspace_bytes_for, for the input gradient. */
+size_t amsim_convam_input_grad_workspace_bytes_for(amsim_lut_t lut, int batch, int input_rows, int input_cols,
+                                                   int in_depth, int filter_rows, int filter_cols, int out_depth,
+                                                   int stride_rows, int stride_cols, int pad_top, int pad_left);
 int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_grad_width, int hole_grad_height,
                                 int pad_top, int pad_left, const float *filter, int filter_rows,
                                 int filter_cols, int out_depth, int stride_rows, int stride_cols, int batch,

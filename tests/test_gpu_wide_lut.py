@@ -31,8 +31,13 @@ def luts():
 
     def get(kind, m):
         if (kind, m) not in cache:
+            import approxtrain_amd
             img = cpu.lutgen32(kind, m)
-            cache[(kind, m)] = (ApproxMulLut.from_entries(_legacy(img), m), img)
+            lut = ApproxMulLut.from_entries(_legacy(img), m)
+            # whole reductions for calls through these handles: the row-staged engine never splits one,
+            # and shapes it does not take then stay bit-comparable too
+            assert approxtrain_amd.load_library().amsim_lut_set_split_k(lut.handle, 0) == 0
+            cache[(kind, m)] = (lut, img)
         return cache[(kind, m)]
     return get
 
@@ -135,11 +140,65 @@ def test_smaller_workspace_falls_back_to_global_gathers(luts):
         ws = torch.empty(nbytes + 256, dtype=torch.uint8, device="cuda")
         wsp = C.c_void_p(ws.data_ptr() + (-ws.data_ptr()) % 256)
         out = torch.empty((M, N), device="cuda")
-        lib.amsim_lut_set_split_k(lut.handle, 0)
         check(lib.amsim_gemm_f32(lut.handle, 0, 0, 0, M, N, K, C.c_void_p(Ad.data_ptr()), K, C.c_void_p(Bd.data_ptr()), N,
                                  C.c_void_p(out.data_ptr()), N, 1, 0, 0, 0, wsp, nbytes, None))
-        lib.amsim_lut_set_split_k(lut.handle, -1)
         outs.append(host(out))
     want = cpu.gemm(img, 11, A, B)
     assert np.array_equal(outs[0].view(np.uint32), want.view(np.uint32))
     assert np.array_equal(outs[1].view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("kind,m", [("MBM", 11), ("MIT", 9)])
+@pytest.mark.parametrize("shape", [((2, 24, 26, 8), (3, 3, 8, 20), (1, 1), "SAME"),
+                                   ((1, 40, 40, 3), (5, 4, 3, 7), (1, 1), "VALID"),
+                                   ((3, 30, 30, 16), (3, 3, 16, 12), (2, 2), "SAME"),
+                                   ((2, 33, 31, 4), (2, 3, 4, 9), (2, 1), "VALID")])
+def test_convolution_forward_and_input_gradient_on_row_staged_engine(luts, kind, m, shape):
+    """Wide tables through the convolution entry points: with the table-aware workspace query the
+    forward pass and the input gradient (all its stride phases with 1024 or more pixels) gather from
+    an im2col staged for the row-staged engine; bit-equal to the oracle's loop nests either way."""
+    from approxtrain_amd import functors
+    lut, img = luts(kind, m)
+    xs, ws, st, padding = shape
+    rng = np.random.default_rng(m * 100 + xs[1] + ws[0])
+    x = rng.standard_normal(xs).astype(np.float32)
+    x[rng.random(xs) < 0.3] = 0.0
+    w = rng.standard_normal(ws).astype(np.float32)
+    y = host(functors.convam(lut, dev(x), dev(w), st, padding))
+    want = cpu.conv2d_fwd(img, m, x, w, st, padding)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    dy = rng.standard_normal(want.shape).astype(np.float32)
+    dx = host(functors.convam_input_grad(lut, xs, dev(w), dev(dy), st, padding))
+    want_dx = cpu.conv2d_grad_input(img, m, xs, w, dy, st, padding)
+    assert np.array_equal(dx.view(np.uint32), want_dx.view(np.uint32))
+
+
+def test_table_aware_convolution_query_adds_the_staged_operand_only_for_wide_tables(luts):
+    import approxtrain_amd
+    from approxtrain_amd import ApproxMulLut
+    from tests.util import lut_path
+    lib = approxtrain_amd.load_library()
+    wide, _ = luts("MBM", 11)
+    narrow = ApproxMulLut(lut_path("MBM", 7))
+    args = (4, 56, 56, 64, 3, 3, 64)
+    base = lib.amsim_convam_workspace_bytes(*args)
+    assert lib.amsim_convam_workspace_bytes_for(narrow.handle, *args) == base
+    assert lib.amsim_convam_workspace_bytes_for(wide.handle, *args) >= (4 * 56 * 56) * 576 * 4   # rows x reduction x 4 bytes: the im2col
+    assert lib.amsim_convam_workspace_bytes_for(None, *args) == base
+
+
+def test_batched_products_on_row_staged_engine(luts):
+    """Strided batches with 1024 or more rows per item, per-item and shared second operands."""
+    from approxtrain_amd import functors
+    lut, img = luts("MIT", 11)
+    rng = np.random.default_rng(31)
+    A = rng.standard_normal((3, 1100, 40)).astype(np.float32)
+    B = rng.standard_normal((3, 40, 18)).astype(np.float32)
+    got = host(functors.gemm(lut, dev(A), dev(B)))
+    for i in range(3):
+        want = cpu.gemm(img, 11, A[i], B[i])
+        assert np.array_equal(got[i].view(np.uint32), want.view(np.uint32))
+    got = host(functors.gemm(lut, dev(A), dev(B[1])))
+    for i in range(3):
+        want = cpu.gemm(img, 11, A[i], B[1])
+        assert np.array_equal(got[i].view(np.uint32), want.view(np.uint32))

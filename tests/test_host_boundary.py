@@ -110,7 +110,7 @@ def test_no_entry_point_crashes_on_null_or_odd_arguments():
                 else:
                     vals.append(None)
             out = getattr(lib, name)(*vals)
-            if name.endswith("_workspace_bytes"):
+            if name.endswith("_workspace_bytes") or name.endswith("_workspace_bytes_for"):
                 assert out >= 0 and (fill > 0 or out == 0), (name, fill, out)
             else:
                 assert out == 1, (name, fill, out)                      # AMSIM_ERR_INVALID: nothing was launched
