@@ -38,7 +38,8 @@ namespace {
 constexpr int WIDE_TILE_ROWS = 4096;              // rows per workgroup (half of that when workgroups are too few, below)
 constexpr int WIDE_TN = 8;                        // columns per workgroup: half a tile of the pre-decoded operand
 constexpr int WIDE_THREADS = WIDE_TN * 64;
-constexpr int WIDE_SLOT_BYTES = 4096;             // LDS bytes reserved per staged table row (2^11 entries x 2)
+constexpr int WIDE_ENTRY_BYTES = WIDE_TN * 2;      // LDS bytes per lane-mantissa value: one 16-bit entry of each staged row
+constexpr int WIDE_BUF_BYTES = 2048 * WIDE_ENTRY_BYTES;  // one stage's rows, interleaved (2^11 mantissa values)
 constexpr int PT_ROWS = 64;                       // rows per workgroup of the transposing pre-pass
 
 struct PTArgs {
@@ -93,26 +94,52 @@ __device__ __forceinline__ uint32_t lds_addr(const void *p)
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
 
-// The 8 entries at addr + j * 4 KB (one per staged table row), issued back to back and waited for
-// together.  Written as one block so that the gathers of a row group stay 8 registers wide (left to
-// itself the scheduler hoists all 64 of a stage and spills accumulators), and so that the compiler
-// does not order them behind the direct-to-LDS copies in flight for the next stage, which write the
-// other half of the buffer.
-__device__ __forceinline__ void gather8(uint32_t addr, uint32_t (&e)[8])
+// The 8 products of one row with the 8 staged entries in e (two per dword), accumulated in place:
+//   factor = (entry << 8) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly, in one
+//   instruction (16-bit multiply by 256 of the dword's low or high half, 32-bit add);
+//   acc += p_pow2 * factor, fused.
+// Written out so that no multiply-add reads a factor written by the instruction just before it (that
+// pairing costs a wait state each time) and so that the two temporaries stay two.
+__device__ __forceinline__ void mac8(float (&acc)[8], const uint4 &e, float ta, uint32_t c256, const uint32_t (&q)[8])
 {
-    asm volatile(
-        "ds_read_u16 %0, %8\n\t"
-        "ds_read_u16 %1, %8 offset:4096\n\t"
-        "ds_read_u16 %2, %8 offset:8192\n\t"
-        "ds_read_u16 %3, %8 offset:12288\n\t"
-        "ds_read_u16 %4, %8 offset:16384\n\t"
-        "ds_read_u16 %5, %8 offset:20480\n\t"
-        "ds_read_u16 %6, %8 offset:24576\n\t"
-        "ds_read_u16 %7, %8 offset:28672\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(e[0]), "=&v"(e[1]), "=&v"(e[2]), "=&v"(e[3]), "=&v"(e[4]), "=&v"(e[5]), "=&v"(e[6]), "=&v"(e[7])
-        : "v"(addr)
-        : "memory");
+    uint32_t t0, t1;
+    asm("v_mad_u32_u16 %[t0], %[ex], %[c], %[q0]\n\t"
+        "v_mad_u32_u16 %[t1], %[ex], %[c], %[q1] op_sel:[1,0,0,0]\n\t"
+        "v_fmac_f32 %[a0], %[ta], %[t0]\n\t"
+        "v_mad_u32_u16 %[t0], %[ey], %[c], %[q2]\n\t"
+        "v_fmac_f32 %[a1], %[ta], %[t1]\n\t"
+        "v_mad_u32_u16 %[t1], %[ey], %[c], %[q3] op_sel:[1,0,0,0]\n\t"
+        "v_fmac_f32 %[a2], %[ta], %[t0]\n\t"
+        "v_mad_u32_u16 %[t0], %[ez], %[c], %[q4]\n\t"
+        "v_fmac_f32 %[a3], %[ta], %[t1]\n\t"
+        "v_mad_u32_u16 %[t1], %[ez], %[c], %[q5] op_sel:[1,0,0,0]\n\t"
+        "v_fmac_f32 %[a4], %[ta], %[t0]\n\t"
+        "v_mad_u32_u16 %[t0], %[ew], %[c], %[q6]\n\t"
+        "v_fmac_f32 %[a5], %[ta], %[t1]\n\t"
+        "v_mad_u32_u16 %[t1], %[ew], %[c], %[q7] op_sel:[1,0,0,0]\n\t"
+        "v_fmac_f32 %[a6], %[ta], %[t0]\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32 %[a7], %[ta], %[t1]"
+        : [a0] "+v"(acc[0]), [a1] "+v"(acc[1]), [a2] "+v"(acc[2]), [a3] "+v"(acc[3]), [a4] "+v"(acc[4]),
+          [a5] "+v"(acc[5]), [a6] "+v"(acc[6]), [a7] "+v"(acc[7]), [t0] "=&v"(t0), [t1] "=&v"(t1)
+        : [ex] "v"(e.x), [ey] "v"(e.y), [ez] "v"(e.z), [ew] "v"(e.w), [ta] "v"(ta), [c] "v"(c256),
+          [q0] "s"(q[0]), [q1] "s"(q[1]), [q2] "s"(q[2]), [q3] "s"(q[3]), [q4] "s"(q[4]), [q5] "s"(q[5]),
+          [q6] "s"(q[6]), [q7] "s"(q[7]));
+}
+
+// Buffer addressing for the streams of the main loop: a load names a resource (uniform base), a
+// uniform byte offset in a scalar register and a 32-bit lane offset, and the hardware adds them --
+// no vector instruction is spent on addresses, and none of the 64-bit vector pointers that flat
+// addressing would keep alive.  Raw buffers of the maximum extent: offsets are not range-checked
+// short of 4 GB.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *uniform_base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(uniform_base), 0, -1, 0x00020000);
+}
+__device__ __forceinline__ uint32_t load_u32(rsrc_t r, uint32_t lane_offset, uint32_t uniform_offset)
+{
+    return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_offset, (int)uniform_offset, 0);
 }
 
 struct WArgs {
@@ -133,22 +160,19 @@ struct WArgs {
     unsigned X, Y;           // row tiles, column strips (blockIdx.y runs over the batch)
 };
 
-// PARTS: KB of a table row copied per stage and slot (4 at width 11, 2 at width 10, 1 below: the copy
-// of a narrower row runs on into the rows behind it, which the image's padding keeps in bounds).
+// MPT: pairs of lane-mantissa values each thread stages per reduction step (2 at width 11: 2048 values
+// over 512 threads; 1 below, where the wavefronts past the row's end stage nothing).
 // RPT: rows per thread, 8 (4096 rows per workgroup: 1 byte of table row pulled per product) or 4 (2048
 // rows, 2 bytes per product: for problems that would otherwise leave compute units without a workgroup).
-template <int PARTS, int RPT>
+template <int MPT, int RPT>
 __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
 {
     constexpr int TILE_ROWS = WIDE_THREADS * RPT;
-    constexpr int WIDE_BUF_BYTES = WIDE_TN * WIDE_SLOT_BYTES;
-    // Two halves of 8 slots x 4 KB, as two objects: the compiler then knows that the direct-to-LDS
-    // copies into one half do not alias the gathers from the other, and does not make the gathers
-    // wait for the copies.
+    // Two halves, as two objects: the compiler then knows that the stores that stage one half do not
+    // alias the gathers from the other, and does not order one behind the other.
     __shared__ __align__(16) uint8_t rows_a[WIDE_BUF_BYTES];
     __shared__ __align__(16) uint8_t rows_b[WIDE_BUF_BYTES];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // Each XCD (private L2) gets a contiguous run of column strips of one row tile: its
     // workgroups then stream the same transposed lane operand.
     unsigned bx, by;
@@ -163,43 +187,71 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     const int64_t row0 = (int64_t)bx * TILE_ROWS;
     const int j0 = by * WIDE_TN;
     constexpr int STRIPS_PER_TILE = QT / WIDE_TN;
-    const int m = a.m, mshift = 23 - m;
-    const uint32_t mmask = (1u << m) - 1u;
+    const int m = a.m, oshift = 23 - m - 4;           // lane mantissa -> byte offset of its 16-byte group
+    const uint32_t omask = ((1u << m) - 1u) << 4;
     const int Kp = a.nchunks * KC;
     const int bz = blockIdx.y, qb = a.q_batches > 1 ? bz : 0;
     const size_t qt_index = (size_t)qb * (a.Jp / QT) + by / STRIPS_PER_TILE;  // tile of the pre-decoded operand
     const cq1_t qtile = (cq1_t)(uintptr_t)(a.qw + qt_index * Kp * QT + (by % STRIPS_PER_TILE) * WIDE_TN);
     const cq1_t qfl = (cq1_t)(uintptr_t)(a.qflags + qt_index * a.nchunks);
-    const uint32_t *pcol = a.pt + (size_t)bz * Kp * a.Rp + row0 + tid;
+    const uint32_t *ptile = a.pt + (size_t)bz * Kp * a.Rp + row0;  // [k][this workgroup's rows]
+    const uint32_t voff = (uint32_t)tid * 4u;                        // this thread's byte offset in a run of dwords
+    const rsrc_t lut_rsrc = make_rsrc(a.lut16);
     const int64_t G = a.Rp / PT_ROWS;
     const uint32_t *pfl = a.pflags + (size_t)bz * a.nchunks * G;
+    uint32_t c256 = 256u;
+    asm volatile("" : "+v"(c256));  // stays in a vector register (the factor instruction has one scalar port)
     float acc[RPT][WIDE_TN];
 #pragma unroll
     for (int rr = 0; rr < RPT; ++rr)
 #pragma unroll
         for (int j = 0; j < WIDE_TN; ++j) acc[rr][j] = 0.0f;
 
-    // wavefront w copies the table row of column j0 + w for stage k into half `buf`
-    auto fill = [&](int k, uint8_t *half) {
-        const uint32_t w = qtile[k * QT + wave];
-        const uint8_t *src = a.lut16 + (size_t)(w & 0x7fffffu) * 2 + lane * 16;
-        uint8_t *dst = half + wave * WIDE_SLOT_BYTES;
+    // Staging of one reduction step's 8 table rows, interleaved: the entries of the 8 rows at lane
+    // mantissa `ma` lie side by side at byte ma * 16, so that ONE 16-byte LDS read serves a row's 8
+    // products (eight scattered 2-byte gathers would meet eight rounds of random bank conflicts).
+    // A thread fetches the dwords (two adjacent entries) at pair index tid (+ 512) of each of the 8
+    // rows, fully coalesced, ...
+    uint32_t tl[MPT][WIDE_TN];
+    // (a row of a table narrower than 10 bits is shorter than one pass of the workgroup: whole
+    // wavefronts then have nothing to stage; rows are multiples of a wavefront's 256 bytes)
+    const bool stages = MPT > 1 || (uint32_t)__builtin_amdgcn_readfirstlane(tid) * 4u < (2u << m);
+    auto fetch_row = [&](int k, int j) {
+        const uint32_t row = (qtile[k * QT + j] & 0x7fffffu) * 2u;  // byte offset of the row q(k, j0 + j) selects
+        if (stages) {
 #pragma unroll
-        for (int part = 0; part < PARTS; ++part) {  // every lane, every part: no branch inside a stage
-#if defined(__HIP_DEVICE_COMPILE__)  // the builtin exists in the device pass only
-            __builtin_amdgcn_global_load_lds(src + part * 1024, dst + part * 1024, 16, 0, 0);
-#endif
+            for (int i = 0; i < MPT; ++i) tl[i][j] = load_u32(lut_rsrc, voff + i * (WIDE_THREADS * 4), row);
+        }
+    };
+    auto fetch_rows = [&](int k) {
+#pragma unroll
+        for (int j = 0; j < WIDE_TN; ++j) fetch_row(k, j);
+    };
+    // ... and regroups them into the 16-byte groups of its two mantissa values (low halves, high halves).
+    auto store_rows = [&](uint8_t *half) {
+        if (!stages) return;
+#pragma unroll
+        for (int i = 0; i < MPT; ++i) {
+            uint4 lo, hi;
+            lo.x = __builtin_amdgcn_perm(tl[i][1], tl[i][0], 0x05040100u); hi.x = __builtin_amdgcn_perm(tl[i][1], tl[i][0], 0x07060302u);
+            lo.y = __builtin_amdgcn_perm(tl[i][3], tl[i][2], 0x05040100u); hi.y = __builtin_amdgcn_perm(tl[i][3], tl[i][2], 0x07060302u);
+            lo.z = __builtin_amdgcn_perm(tl[i][5], tl[i][4], 0x05040100u); hi.z = __builtin_amdgcn_perm(tl[i][5], tl[i][4], 0x07060302u);
+            lo.w = __builtin_amdgcn_perm(tl[i][7], tl[i][6], 0x05040100u); hi.w = __builtin_amdgcn_perm(tl[i][7], tl[i][6], 0x07060302u);
+            uint4 *dst = reinterpret_cast<uint4 *>(half + (size_t)(tid + i * WIDE_THREADS) * (2 * WIDE_ENTRY_BYTES));
+            dst[0] = lo;
+            dst[1] = hi;
         }
     };
     uint32_t pc[RPT], pn[RPT];
     auto load_p = [&](int k, uint32_t (&dst)[RPT]) {
+        const rsrc_t src = make_rsrc(ptile + (size_t)k * a.Rp);
 #pragma unroll
-        for (int rr = 0; rr < RPT; ++rr) dst[rr] = pcol[(size_t)k * a.Rp + rr * WIDE_THREADS];
+        for (int rr = 0; rr < RPT; ++rr) dst[rr] = load_u32(src, voff, rr * (WIDE_THREADS * 4));
     };
 
-    fill(0, rows_a);
+    fetch_rows(0);
     load_p(0, pc);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    store_rows(rows_a);
     __syncthreads();
 
     // Is any chunk of this workgroup's tile flagged (by its column tile or by a 64-row group of its
@@ -213,30 +265,27 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
                                  i % (TILE_ROWS / PT_ROWS)];
     tile_flagged = __syncthreads_or(tile_flagged);
 
-    // one stage: copies for stage k + 1 go into `next` while stage k gathers from `cur`
+    // one stage: the rows of stage k + 1 are fetched while stage k gathers from `cur`, and regrouped
+    // into `next` once its products are done
     auto stage = [&](auto exact_tag, int k, const uint8_t *cur, uint8_t *next) {
         constexpr bool EXACT = decltype(exact_tag)::value;
-        // (the last stage copies its own rows and operands once more instead of branching: a
+        // (the last stage fetches its own rows and operands once more instead of branching: a
         // straight-line stage keeps the compiler from sinking one stage's FMAs into the next)
         const int kn = min(k + 1, Kp - 1);
-        fill(kn, next);  // everyone left that half at the barrier that ended the stage before
-        load_p(kn, pn);
         if constexpr (!EXACT) {
             uint32_t qt[WIDE_TN];
 #pragma unroll
             for (int j = 0; j < WIDE_TN; ++j) qt[j] = qtile[k * QT + j] & 0xff800000u;
+            fetch_rows(kn);
+            load_p(kn, pn);
 #pragma unroll
             for (int rr = 0; rr < RPT; ++rr) {
-                const float ta = u2f(pc[rr] & 0xff800000u);
-                const uint32_t off = ((pc[rr] >> mshift) & mmask) << 1;
-                uint32_t e[WIDE_TN];
-                gather8(lds_addr(cur) + off, e);
-#pragma unroll
-                for (int j = 0; j < WIDE_TN; ++j)
-                    // (entry << 8) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly
-                    acc[rr][j] = __builtin_fmaf(ta, u2f((e[j] << 8) + qt[j]), acc[rr][j]);
+                const uint4 e = *reinterpret_cast<const uint4 *>(cur + ((pc[rr] >> oshift) & omask));
+                mac8(acc[rr], e, u2f(pc[rr] & 0xff800000u), c256, qt);
             }
         } else {
+            fetch_rows(kn);
+            load_p(kn, pn);
             // Rare: full-domain product; q's raw bits come from where the operand lies.  The
             // accumulators take a detour through private memory so that this loop can index them
             // dynamically (small code, one product at a time) while the fast path keeps them in
@@ -255,8 +304,8 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
             for (int idx = 0; idx < RPT * WIDE_TN; ++idx) {
                 const int rr = idx / WIDE_TN, j = idx % WIDE_TN;
                 const uint32_t raw = praw[rr];
-                const uint32_t off = ((raw >> mshift) & mmask) << 1;
-                const uint32_t e16 = (uint32_t)*reinterpret_cast<const uint16_t *>(cur + off + j * WIDE_SLOT_BYTES) << 8;
+                const uint32_t off = (raw >> oshift) & omask;
+                const uint32_t e16 = (uint32_t)*reinterpret_cast<const uint16_t *>(cur + off + j * 2) << 8;
                 const uint32_t qr = q_raw_bits(qd, qsrc, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)k, (uint32_t)(j0 + j));
                 tmp[idx] += a.lane_first ? am_exact(raw, qr, e16) : am_exact(qr, raw, e16);
             }
@@ -267,10 +316,10 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         }
 #pragma unroll
         for (int rr = 0; rr < RPT; ++rr) pc[rr] = pn[rr];
-        // my copies for the next stage have landed; after the barrier so have everyone's, and
-        // every wavefront is done gathering from this stage's half
+        // everyone left `next` at the barrier that ended the stage before; after this one everyone's
+        // groups have landed and every wavefront is done gathering from `cur`
         __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        store_rows(next);
         __syncthreads();
     };
     if (!tile_flagged) {
@@ -377,14 +426,11 @@ int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_
     const int64_t total = (int64_t)wa.X * wa.Y;
     if (total >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "workgroup count exceeds the grid limit");
     const dim3 grid((unsigned)total, (unsigned)d.batch);
-    const int parts = lut.m >= 11 ? 4 : lut.m == 10 ? 2 : 1;
     if (half) {
-        if (parts == 4) lutgemm_wide_kernel<4, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
-        else if (parts == 2) lutgemm_wide_kernel<2, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        if (lut.m >= 11) lutgemm_wide_kernel<2, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
         else lutgemm_wide_kernel<1, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
     } else {
-        if (parts == 4) lutgemm_wide_kernel<4, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
-        else if (parts == 2) lutgemm_wide_kernel<2, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        if (lut.m >= 11) lutgemm_wide_kernel<2, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
         else lutgemm_wide_kernel<1, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
     }
     AMSIM_HIP_CHECK(hipGetLastError());
