@@ -17,6 +17,8 @@ constexpr int MICRO_UNROLL = 16;
 //       4: a 4-op mix (add, mul, lshl_add, fma)
 //       5: the GEMM's mix per pair of MACs: one v_lshl_add_u64 (VGPR pair + SGPR pair, two LUT
 //          addresses), two v_lshl_add_u32 (VGPR << 16 + SGPR), two v_fma_f32 -- 5 ops per two slots
+//       6: the row-staged GEMM's pair per product: v_mad_u32_u16 (16-bit half * 256 + SGPR) feeding a
+//          v_fma_f32 two instructions later -- 2 ops per slot
 template <int VMODE>
 __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, float *sink, long long *clk)
 {
@@ -42,6 +44,14 @@ __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, fl
                 asm volatile("v_lshl_add_u64 %0, %1, 0, %2" : "=v"(t2) : "v"(pair), "s"(spair));
                 asm volatile("v_lshl_add_u32 %0, %1, 16, %2" : "=v"(t0) : "v"((uint32_t)t2), "s"(iters));
                 asm volatile("v_lshl_add_u32 %0, %1, 16, %2" : "=v"(t1) : "v"((uint32_t)(t2 >> 32)), "s"(iters));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j]) : "v"(c2), "v"(t0));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j + 1]) : "v"(c2), "v"(t1));
+            } else if (VMODE == 6) {
+                if (j & 1) continue;
+                uint32_t t0, t1;
+                asm volatile("v_mad_u32_u16 %0, %2, %3, %4\n\t"
+                             "v_mad_u32_u16 %1, %2, %3, %4 op_sel:[1,0,0,0]"
+                             : "=&v"(t0), "=&v"(t1) : "v"((uint32_t)pair), "v"(c1), "s"(iters));
                 asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j]) : "v"(c2), "v"(t0));
                 asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j + 1]) : "v"(c2), "v"(t1));
             } else {
@@ -155,6 +165,10 @@ __global__ __launch_bounds__(MICRO_THREADS, 6) void micro_lds_fit_kernel(int ite
 //   WMODE 3: both together, the shape of the row-staged GEMM: per stage a 1024-thread workgroup
 //            pulls 16 rows (64 KB) into one half of its LDS while every thread gathers 64
 //            entries from the other half and feeds them to the convert + FMA pair
+//   WMODE 4: ds_read_b128 with the lanes scattered over the 2048 16-byte groups of a 32 KB half (the
+//            interleaved layout: one read brings the entries of 8 rows); counts 8 products per read
+//   WMODE 5: rows pulled into registers by coalesced 4-byte loads (16 per thread and stage, buffer
+//            addressing), nothing else: the bytes per second the register path brings in
 // ---------------------------------------------------------------------------
 constexpr int WIDE_THREADS = 1024;
 constexpr int WIDE_ROW_BYTES = 4096;
@@ -220,6 +234,40 @@ __global__ __launch_bounds__(WIDE_THREADS) void micro_wide_kernel(const uint8_t 
         for (int i = tid; i < 2 * WIDE_ROWS * WIDE_ROW_BYTES / 4; i += WIDE_THREADS) reinterpret_cast<uint32_t *>(wl)[i] = mix32(i) & 0x7fff7fffu;
         __syncthreads();
         for (int it = 0; it < iters; ++it) gather(it & 1, (uint32_t)it * 2u);
+    } else if (WMODE == 4) {
+        for (int i = tid; i < 2 * WIDE_ROWS * WIDE_ROW_BYTES / 4; i += WIDE_THREADS) reinterpret_cast<uint32_t *>(wl)[i] = mix32(i);
+        __syncthreads();
+        uint32_t x = 0;
+        for (int it = 0; it < iters; ++it) {
+            const uint8_t *base = wl + (it & 1) * 32768;
+#pragma unroll
+            for (int rr = 0; rr < 8; ++rr) {
+                const uint32_t off = (mix32(lane_off + rr * 7919u + (uint32_t)it) & 2047u) * 16u;
+                const uint4 e = *reinterpret_cast<const uint4 *>(base + off);
+                x ^= e.x ^ e.y ^ e.z ^ e.w;
+            }
+        }
+        if (x == 0x12345u) sink[tid & 255] = 1.0f;  // (an integer-valued float could never equal the sentinel below)
+    } else if (WMODE == 5) {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(table), 0, -1, 0x00020000);
+        uint32_t x = 0, va[WIDE_ROWS], vb[WIDE_ROWS];
+        auto pull = [&](int it, uint32_t (&v)[WIDE_ROWS]) {
+#pragma unroll
+            for (int j = 0; j < WIDE_ROWS; ++j) {
+                const uint32_t row = mix32((uint32_t)it * 977u + blockIdx.x * 131u + j) % table_rows;
+                v[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, tid * 4, (int)(row * WIDE_ROW_BYTES), 0);
+            }
+        };
+        pull(0, va);
+        for (int it = 0; it < iters; it += 2) {  // one stage's loads are in flight while the stage before is consumed
+            pull(it + 1, vb);
+#pragma unroll
+            for (int j = 0; j < WIDE_ROWS; ++j) x ^= va[j];
+            pull(it + 2, va);
+#pragma unroll
+            for (int j = 0; j < WIDE_ROWS; ++j) x ^= vb[j];
+        }
+        if (x == 0x12345u) sink[tid & 255] = 1.0f;  // (an integer-valued float could never equal the sentinel below)
     } else {
         fill(0, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -263,7 +311,7 @@ int amsim_calibration_copy(const float *src, float *dst, size_t n, void *stream)
 }
 
 // Runs micro-kernel `kind` (0 = VALU FMA, 1..6 = LDS gather modes 0..5,
-// 10..15 = VALU modes 0..5 with `sink[512..]` receiving, as two 64-bit counts, the
+// 10..16 = VALU modes 0..6 with `sink[512..]` receiving, as two 64-bit counts, the
 // shader-clock ticks of one workgroup's loop and the same interval in 100 MHz ticks,
 // 21 / 22 = byte gathers inside a row / scattered at the LUT GEMM's own LDS footprint and
 // occupancy) with
@@ -274,7 +322,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
                      double *ops_per_launch)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (kind < 0 || (kind > 6 && kind < 10) || (kind > 15 && kind < 21) || kind > 22 || blocks < 1 || iters < 1 || reps < 1 || !sink || !ms_per_launch || !ops_per_launch)
+    if (kind < 0 || (kind > 6 && kind < 10) || (kind > 16 && kind < 21) || kind > 22 || blocks < 1 || iters < 1 || reps < 1 || !sink || !ms_per_launch || !ops_per_launch)
         return fail(AMSIM_ERR_INVALID, "bad microbench arguments");
     hipEvent_t e0, e1;
     AMSIM_HIP_CHECK(hipEventCreate(&e0));
@@ -288,6 +336,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
         case 13: micro_valu_kernel<3><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 14: micro_valu_kernel<4><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 15: micro_valu_kernel<5><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
+        case 16: micro_valu_kernel<6><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 21: micro_lds_fit_kernel<0><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
         case 22: micro_lds_fit_kernel<1><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
         case 1: micro_lds_kernel<0><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
@@ -309,20 +358,20 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
     AMSIM_HIP_CHECK(hipEventDestroy(e1));
     AMSIM_HIP_CHECK(hipGetLastError());
     *ms_per_launch = (double)ms / reps;
-    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4.0 : kind == 15 ? 2.5 : 1.0);
+    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4.0 : kind == 15 ? 2.5 : kind == 16 ? 2.0 : 1.0);
     return AMSIM_OK;
 }
 
 
-// Micro-kernels for tables too wide for the LDS (kinds 0..3 = WMODE above).  `table` is any
+// Micro-kernels for tables too wide for the LDS (kinds 0..5 = WMODE above).  `table` is any
 // device buffer of table_bytes >= 8 KB (rows of 4 KB are read from it), `blocks` workgroups of
 // 1024 threads (kind 0: 16 wavefronts each), `iters` stages of 16 rows.  ops_per_launch counts
-// products (kinds 0, 2, 3) or bytes pulled into LDS (kind 1; kind 3 pulls 1 byte per product).
+// products (kinds 0, 2, 3, 4) or bytes pulled in (kinds 1, 5; kind 3 pulls 1 byte per product).
 int amsim_microbench_wide(int kind, int blocks, int iters, int reps, void *stream_, const void *table, size_t table_bytes,
                           float *sink, double *ms_per_launch, double *ops_per_launch)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (kind < 0 || kind > 3 || blocks < 1 || iters < 1 || reps < 1 || !table || table_bytes < 2 * WIDE_ROW_BYTES ||
+    if (kind < 0 || kind > 5 || blocks < 1 || iters < 1 || reps < 1 || !table || table_bytes < 2 * WIDE_ROW_BYTES ||
         ((uintptr_t)table & 15) || !sink || !ms_per_launch || !ops_per_launch)
         return fail(AMSIM_ERR_INVALID, "bad microbench arguments");
     const uint32_t rows = (uint32_t)std::min<size_t>(table_bytes / WIDE_ROW_BYTES, 1u << 20);
@@ -332,11 +381,14 @@ int amsim_microbench_wide(int kind, int blocks, int iters, int reps, void *strea
     AMSIM_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(micro_wide_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     AMSIM_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(micro_wide_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     AMSIM_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(micro_wide_kernel<3>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    AMSIM_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(micro_wide_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     auto launch = [&]() {
         switch (kind) {
         case 0: micro_wide_kernel<0><<<blocks, WIDE_THREADS, 0, stream>>>(t, rows, iters, sink); break;
         case 1: micro_wide_kernel<1><<<blocks, WIDE_THREADS, lds, stream>>>(t, rows, iters, sink); break;
         case 2: micro_wide_kernel<2><<<blocks, WIDE_THREADS, lds, stream>>>(t, rows, iters, sink); break;
+        case 4: micro_wide_kernel<4><<<blocks, WIDE_THREADS, lds, stream>>>(t, rows, iters, sink); break;
+        case 5: micro_wide_kernel<5><<<blocks, WIDE_THREADS, 0, stream>>>(t, rows, iters, sink); break;
         default: micro_wide_kernel<3><<<blocks, WIDE_THREADS, lds, stream>>>(t, rows, iters, sink); break;
         }
     };
@@ -354,8 +406,11 @@ int amsim_microbench_wide(int kind, int blocks, int iters, int reps, void *strea
     AMSIM_HIP_CHECK(hipEventDestroy(e1));
     AMSIM_HIP_CHECK(hipGetLastError());
     *ms_per_launch = (double)ms / reps;
-    const double per_stage = kind == 0 ? (double)WIDE_THREADS * WIDE_ROWS : kind == 1 ? (double)WIDE_ROWS * WIDE_ROW_BYTES
-                                                                                   : (double)WIDE_THREADS * 4 * WIDE_ROWS;
+    const double per_stage = kind == 0   ? (double)WIDE_THREADS * WIDE_ROWS
+                             : kind == 1 ? (double)WIDE_ROWS * WIDE_ROW_BYTES
+                             : kind == 4 ? (double)WIDE_THREADS * 8 * 8
+                             : kind == 5 ? (double)WIDE_THREADS * WIDE_ROWS * 4
+                                         : (double)WIDE_THREADS * 4 * WIDE_ROWS;
     *ops_per_launch = (double)blocks * iters * per_stage;
     return AMSIM_OK;
 }
