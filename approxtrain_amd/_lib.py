@@ -52,6 +52,7 @@ SIGNATURES = {
     "amsim_convam_input_grad_workspace_bytes_for": (_sz, [_p] + [_i] * 11),
     "amsim_convam_input_grad_f32": (_i, [_p, _f, _i, _i, _i, _i, _f] + [_i] * 9 + [_f, _i, _i, _p, _sz, _p]),
     "amsim_convam_filter_grad_workspace_bytes": (_sz, [_i] * 7),
+    "amsim_convam_filter_grad_workspace_bytes_for": (_sz, [_p] + [_i] * 7),
     "amsim_convam_filter_grad_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p, _sz, _p]),
     "amsim_denseam_workspace_bytes": (_sz, [_i] * 3),
     "amsim_denseam_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),

@@ -469,6 +469,17 @@ size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out
     return need;
 }
 
+size_t amsim_convam_filter_grad_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols,
+                                                    int out_depth, int filter_rows, int filter_cols, int in_depth)
+{
+    size_t need = amsim_convam_filter_grad_workspace_bytes(batch, out_rows, out_cols, out_depth, filter_rows,
+                                                           filter_cols, in_depth);
+    if (need && lut != nullptr && lut->l.m > 7 && !(filter_rows == 1 && filter_cols == 1))
+        need = std::max(need, gemm_workspace_bytes_wide((int64_t)filter_rows * filter_cols * in_depth, out_depth,
+                                                        (int64_t)batch * out_rows * out_cols, 1, 1));
+    return need;
+}
+
 int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const float *grad, int input_rows,
                                  int input_cols, int batch, int in_depth, int out_cols, int out_rows,
                                  int out_depth, int filter_left_offset, int filter_top_offset, int stride_rows,

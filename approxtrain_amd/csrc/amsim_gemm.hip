@@ -922,7 +922,7 @@ static size_t unsplit_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
 size_t gemm_workspace_bytes_wide(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 {
     if (R <= 0 || J <= 0 || K <= 0 || batch <= 0 || !wide_shape_eligible(R, batch)) return 0;
-    return unsplit_bytes(R, J, K, batch, q_batches) + wide_workspace_bytes(R, K, batch);
+    return unsplit_bytes(R, J, K, batch, q_batches) + wide_workspace_bytes(R, J, K, batch);
 }
 
 size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
@@ -1024,12 +1024,12 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
                                              std::to_string(need) + " bytes");
     if (use_direct) return run_gemm_direct(lut, d, may_split, workspace, workspace_bytes, stream);
-    if (wide_eligible(lut.m, d)) {
+    if (wide_eligible(lut.m, d, may_split)) {
         // tables too wide for the LDS: the row-staged engine, if the workspace also holds the
         // transposed lane operand (else the global-gather variant below does the job, slowly)
         const Plan pq = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, false, WAVES_PER_SIMD);
         if (workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-            workspace_bytes >= pq.total + wide_workspace_bytes(d.R, d.K, d.batch)) {
+            workspace_bytes >= pq.total + wide_workspace_bytes(d.R, d.J, d.K, d.batch)) {
             uint8_t *ws = static_cast<uint8_t *>(workspace);
             QArgs qa{};
             qa.q = d.q;
@@ -1038,7 +1038,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
             qa.qflags = reinterpret_cast<uint32_t *>(ws + pq.off_flags);
             qa.qdesc_out = reinterpret_cast<QDesc *>(ws + pq.off_qdesc);
             if (const int rc = launch_q_prepass(qa, d.q.batches, stream)) return rc;
-            return run_gemm_wide(lut, d, WideQ{qa.qw, qa.qflags, qa.qdesc_out, pq.Jp, pq.nchunks}, ws + pq.total, stream);
+            return run_gemm_wide(lut, d, WideQ{qa.qw, qa.qflags, qa.qdesc_out, pq.Jp, pq.nchunks}, ws + pq.total, may_split, stream);
         }
     }
     const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, may_split, waves64_of(d.p, d.K));

@@ -158,6 +158,9 @@ struct WArgs {
     int q_batches;           // 1: the uniform operand is shared by every batch item
     Epilogue ep;
     unsigned X, Y;           // row tiles, column strips (blockIdx.y runs over the batch)
+    int nsplit;              // slices of the reduction (blockIdx.z), each a whole number of chunks
+    int chunks_per_split;
+    float *partial;          // nsplit > 1: [nsplit][batch][X * tile rows][Jp] partial sums instead of `out`
 };
 
 // MPT: pairs of lane-mantissa values each thread stages per reduction step (2 at width 11: 2048 values
@@ -190,6 +193,8 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     const int m = a.m, oshift = 23 - m - 4;           // lane mantissa -> byte offset of its 16-byte group
     const uint32_t omask = ((1u << m) - 1u) << 4;
     const int Kp = a.nchunks * KC;
+    const int ch_beg = blockIdx.z * a.chunks_per_split, ch_end = min(ch_beg + a.chunks_per_split, a.nchunks);
+    const int kbeg = ch_beg * KC, kend = ch_end * KC;  // this workgroup's slice of the reduction
     const int bz = blockIdx.y, qb = a.q_batches > 1 ? bz : 0;
     const size_t qt_index = (size_t)qb * (a.Jp / QT) + by / STRIPS_PER_TILE;  // tile of the pre-decoded operand
     const cq1_t qtile = (cq1_t)(uintptr_t)(a.qw + qt_index * Kp * QT + (by % STRIPS_PER_TILE) * WIDE_TN);
@@ -249,8 +254,8 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         for (int rr = 0; rr < RPT; ++rr) dst[rr] = load_u32(src, voff, rr * (WIDE_THREADS * 4));
     };
 
-    fetch_rows(0);
-    load_p(0, pc);
+    fetch_rows(kbeg);
+    load_p(kbeg, pc);
     store_rows(rows_a);
     __syncthreads();
 
@@ -258,10 +263,10 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     // row tile)?  Almost never: then the whole reduction runs the loop nest that holds nothing but
     // fast stages, whose registers the rare path's state cannot crowd.
     int tile_flagged = 0;
-    for (int ch = tid; ch < a.nchunks; ch += WIDE_THREADS)
+    for (int ch = ch_beg + tid; ch < ch_end; ch += WIDE_THREADS)
         tile_flagged |= (int)a.qflags[qt_index * a.nchunks + ch];
-    for (int i = tid; i < a.nchunks * (TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
-        tile_flagged |= (int)pfl[(size_t)(i / (TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (TILE_ROWS / PT_ROWS) +
+    for (int i = tid; i < (ch_end - ch_beg) * (TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
+        tile_flagged |= (int)pfl[(size_t)(ch_beg + i / (TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (TILE_ROWS / PT_ROWS) +
                                  i % (TILE_ROWS / PT_ROWS)];
     tile_flagged = __syncthreads_or(tile_flagged);
 
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         constexpr bool EXACT = decltype(exact_tag)::value;
         // (the last stage fetches its own rows and operands once more instead of branching: a
         // straight-line stage keeps the compiler from sinking one stage's FMAs into the next)
-        const int kn = min(k + 1, Kp - 1);
+        const int kn = min(k + 1, kend - 1);
         if constexpr (!EXACT) {
             uint32_t qt[WIDE_TN];
 #pragma unroll
@@ -324,12 +329,12 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     };
     if (!tile_flagged) {
 #pragma unroll 1
-        for (int k = 0; k < Kp; k += 2) {
+        for (int k = kbeg; k < kend; k += 2) {
             stage(std::false_type{}, k, rows_a, rows_b);
             stage(std::false_type{}, k + 1, rows_b, rows_a);
         }
     } else {
-        for (int ch = 0; ch < a.nchunks; ++ch) {
+        for (int ch = ch_beg; ch < ch_end; ++ch) {
             const uint32_t pf = lane < TILE_ROWS / PT_ROWS ? pfl[(size_t)ch * G + (size_t)bx * (TILE_ROWS / PT_ROWS) + lane] : 0u;
             const bool unsafe = (qfl[ch] != 0u) | (__any(pf != 0u) != 0);
             if (!unsafe) {
@@ -348,6 +353,20 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         }
     }
 
+    if (a.nsplit > 1) {
+        // a slice's sums go to the workspace whole (padding rows and columns included: zeros);
+        // the fixed-order reduction kernel adds the slices and applies the epilogue
+        const int64_t prows = (int64_t)a.X * TILE_ROWS;
+        float *part = a.partial + (((size_t)blockIdx.z * gridDim.y + bz) * prows + row0) * a.Jp + j0;
+#pragma unroll
+        for (int rr = 0; rr < RPT; ++rr) {
+            float4 *o4 = reinterpret_cast<float4 *>(part + (size_t)(rr * WIDE_THREADS + tid) * a.Jp);
+#pragma unroll
+            for (int j = 0; j < WIDE_TN / 4; ++j)
+                o4[j] = make_float4(acc[rr][4 * j], acc[rr][4 * j + 1], acc[rr][4 * j + 2], acc[rr][4 * j + 3]);
+        }
+        return;
+    }
 #pragma unroll
     for (int rr = 0; rr < RPT; ++rr) {
         const int64_t r = row0 + rr * WIDE_THREADS + tid;
@@ -371,36 +390,98 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
 }
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-inline int64_t padded_rows(int64_t R) { return (R + WIDE_TILE_ROWS - 1) / WIDE_TILE_ROWS * WIDE_TILE_ROWS; }
+// Rows of the transposed operand: whole tiles of the height the problem will run with (problems of up
+// to 2048 rows are one tile of 1024 or 2048 rows, so that filter gradients -- a few hundred to a few
+// thousand filter elements over the lanes -- do not pad to 4096).
+inline int64_t padded_rows(int64_t R)
+{
+    if (R <= WIDE_TILE_ROWS / 4) return WIDE_TILE_ROWS / 4;
+    if (R <= WIDE_TILE_ROWS / 2) return WIDE_TILE_ROWS / 2;
+    return (R + WIDE_TILE_ROWS - 1) / WIDE_TILE_ROWS * WIDE_TILE_ROWS;
+}
+
+// How a problem is cut: tile height, and the reduction into nsplit slices of whole chunks when the
+// tiles alone would leave half or more of the workgroup slots (two per compute unit) empty and slices
+// are allowed.
+struct WidePlan {
+    int tile_rows, nsplit, chunks_per_split;
+    int64_t Rp, X, strips, nchunks;
+    size_t pt_bytes, flag_bytes, partial_bytes;
+};
+WidePlan wide_plan(int64_t R, int64_t J, int64_t K, int batch, bool may_split, int cus)
+{
+    WidePlan pl{};
+    pl.Rp = padded_rows(R);
+    pl.nchunks = (K + KC - 1) / KC;
+    pl.strips = (J + QT - 1) / QT * (QT / WIDE_TN);
+    const int64_t slots = 2 * (int64_t)cus;
+    pl.tile_rows = (int)std::min<int64_t>(pl.Rp, WIDE_TILE_ROWS);
+    // half-height tiles when full-height ones would leave slots empty
+    if (pl.tile_rows == WIDE_TILE_ROWS && (pl.Rp / WIDE_TILE_ROWS) * pl.strips * batch < slots) pl.tile_rows = WIDE_TILE_ROWS / 2;
+    pl.X = (R + pl.tile_rows - 1) / pl.tile_rows;
+    const int64_t tiles = pl.X * pl.strips * batch;
+    pl.nsplit = 1;
+    pl.chunks_per_split = (int)pl.nchunks;
+    // (slices of at least 4 chunks = 128 stages, a few hundred microseconds: shorter ones would not
+    // pay for their partial sums and the reduction launch)
+    if (may_split && 2 * tiles <= slots && pl.nchunks >= 16) {
+        const int64_t want = std::min<int64_t>(pl.nchunks / 4, std::min<int64_t>((slots + tiles - 1) / tiles, 65535));
+        pl.chunks_per_split = (int)((pl.nchunks + want - 1) / want);
+        pl.nsplit = (int)((pl.nchunks + pl.chunks_per_split - 1) / pl.chunks_per_split);
+    }
+    pl.pt_bytes = align256((size_t)batch * pl.nchunks * KC * pl.Rp * sizeof(uint32_t));
+    pl.flag_bytes = align256((size_t)batch * pl.nchunks * (pl.Rp / PT_ROWS) * sizeof(uint32_t));
+    const int64_t Jp = pl.strips * WIDE_TN;
+    pl.partial_bytes = pl.nsplit > 1 ? align256((size_t)pl.nsplit * batch * pl.X * pl.tile_rows * Jp * sizeof(float)) : 0;
+    return pl;
+}
+
+template <int RPT>
+void launch_wide(const WArgs &wa, dim3 grid, int m, hipStream_t stream)
+{
+    if (m >= 11) lutgemm_wide_kernel<2, RPT><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+    else lutgemm_wide_kernel<1, RPT><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+}
 
 }  // namespace
 
 bool wide_shape_eligible(int64_t R, int batch) { return batch >= 1 && batch <= 65535 && R >= WIDE_MIN_ROWS; }
 
-// Dense and patch (forward / input-gradient convolution) lane operands; the filter gradient's rows
-// are the few filter elements and its reduction the many pixels, the opposite of what this engine
-// needs, so it stays on the global-gather variant.
-bool wide_eligible(int m, const GemmDesc &d)
+// Dense, patch (forward / input-gradient convolution) and filter-gradient lane operands.  A problem
+// that would run on a handful of workgroups because its reduction may not be sliced (a filter
+// gradient in whole-reduction mode: few rows, very long reduction) is left to the global-gather
+// variant, which at least fills the machine.
+bool wide_eligible(int m, const GemmDesc &d, bool may_split)
 {
-    return m > 7 && (d.p.kind == P_DENSE || d.p.kind == P_PATCH) && wide_shape_eligible(d.R, d.batch);
+    if (m <= 7 || !wide_shape_eligible(d.R, d.batch)) return false;
+    const int cus = device_compute_units();
+    const WidePlan pl = wide_plan(d.R, d.J, d.K, d.batch, may_split, cus);
+    const int64_t wgs = pl.X * pl.strips * d.batch * pl.nsplit;
+    return wgs * 8 >= cus || pl.nchunks <= 64;
 }
 
-size_t wide_workspace_bytes(int64_t R, int64_t K, int batch)
+size_t wide_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch)
 {
-    const int64_t Rp = padded_rows(R), nchunks = (K + KC - 1) / KC;
-    return align256((size_t)batch * nchunks * KC * Rp * sizeof(uint32_t)) +
-           align256((size_t)batch * nchunks * (Rp / PT_ROWS) * sizeof(uint32_t));
+    // the larger of what a sliced and a whole reduction ask for, on any device size
+    size_t need = 0;
+    for (int cus : {device_compute_units(), 256, 304})
+        for (bool split : {false, true}) {
+            const WidePlan pl = wide_plan(R, J, K, batch, split, cus);
+            need = std::max(need, pl.pt_bytes + pl.flag_bytes + pl.partial_bytes);
+        }
+    return need;
 }
 
-int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, hipStream_t stream)
+int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, bool may_split, hipStream_t stream)
 {
-    const int64_t Rp = padded_rows(d.R);
+    const WidePlan pl = wide_plan(d.R, d.J, d.K, d.batch, may_split, device_compute_units());
+    const int64_t Rp = pl.Rp;
     const int64_t G = Rp / PT_ROWS;
     uint8_t *ws = static_cast<uint8_t *>(wide_ws);
     PTArgs pa{};
     pa.p = d.p; pa.R = d.R; pa.K = d.K; pa.Rp = Rp; pa.nchunks = q.nchunks;
     pa.pt = reinterpret_cast<uint32_t *>(ws);
-    pa.pflags = reinterpret_cast<uint32_t *>(ws + align256((size_t)d.batch * q.nchunks * KC * Rp * sizeof(uint32_t)));
+    pa.pflags = reinterpret_cast<uint32_t *>(ws + pl.pt_bytes);
     const int64_t pwgs = G * q.nchunks;
     if (pwgs >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "lane operand exceeds the grid limit");
     p_linear_kernel<<<dim3((unsigned)pwgs, (unsigned)d.batch), WG_THREADS, 0, stream>>>(pa);
@@ -417,23 +498,26 @@ int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_
     wa.vec_store = (d.so_j == 1 && d.so_r % 4 == 0 && d.out_batch_stride % 4 == 0 && ((uintptr_t)d.out & 15) == 0) ? 1 : 0;
     wa.q_batches = d.q.batches;
     wa.ep = Epilogue{d.bias_j, d.bias_r, d.act, d.omap};
-    // half-height tiles when full-height ones would leave workgroup slots (two per compute unit) empty
-    const int64_t strips = q.Jp / WIDE_TN;
-    const bool half = (Rp / WIDE_TILE_ROWS) * strips * d.batch < 2 * (int64_t)device_compute_units();
-    const int tile_rows = half ? WIDE_TILE_ROWS / 2 : WIDE_TILE_ROWS;
-    wa.X = (unsigned)((d.R + tile_rows - 1) / tile_rows);
-    wa.Y = (unsigned)strips;
+    wa.X = (unsigned)pl.X;
+    wa.Y = (unsigned)(q.Jp / WIDE_TN);
+    wa.nsplit = pl.nsplit;
+    wa.chunks_per_split = pl.chunks_per_split;
+    wa.partial = reinterpret_cast<float *>(ws + pl.pt_bytes + pl.flag_bytes);
     const int64_t total = (int64_t)wa.X * wa.Y;
     if (total >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "workgroup count exceeds the grid limit");
-    const dim3 grid((unsigned)total, (unsigned)d.batch);
-    if (half) {
-        if (lut.m >= 11) lutgemm_wide_kernel<2, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
-        else lutgemm_wide_kernel<1, 4><<<grid, WIDE_THREADS, 0, stream>>>(wa);
-    } else {
-        if (lut.m >= 11) lutgemm_wide_kernel<2, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
-        else lutgemm_wide_kernel<1, 8><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+    const dim3 grid((unsigned)total, (unsigned)d.batch, (unsigned)pl.nsplit);
+    switch (pl.tile_rows / WIDE_THREADS) {
+    case 8: launch_wide<8>(wa, grid, lut.m, stream); break;
+    case 4: launch_wide<4>(wa, grid, lut.m, stream); break;
+    default: launch_wide<2>(wa, grid, lut.m, stream); break;
     }
     AMSIM_HIP_CHECK(hipGetLastError());
+    if (pl.nsplit > 1) {
+        RArgs ra{wa.partial, d.out, d.R, d.J, pl.X * pl.tile_rows, d.so_r, d.so_j, d.out_batch_stride, q.Jp, pl.nsplit,
+                 d.batch, 0, wa.ep};
+        launch_reduce(ra, stream);
+        AMSIM_HIP_CHECK(hipGetLastError());
+    }
     return AMSIM_OK;
 }
 

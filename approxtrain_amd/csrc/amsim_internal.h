@@ -121,11 +121,11 @@ void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, b
 int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream);
 
 // ---- the row-staged engine for tables too wide for the LDS (mantissa widths 8..11) ----------
-// Serves dense and patch (convolution forward / input gradient) problems with at least
-// WIDE_MIN_ROWS rows per batch item when the caller's workspace also holds the transposed lane
-// operand (wide_workspace_bytes on top of the unsplit plan); everything else with such tables
-// runs on the LDS-table engine's global-gather variant.
-constexpr int64_t WIDE_MIN_ROWS = 1024;
+// Serves problems with at least WIDE_MIN_ROWS rows per batch item (dense, convolution patches,
+// filter-gradient gathers) when the caller's workspace also holds the transposed lane operand and
+// the partial sums of a sliced reduction (wide_workspace_bytes on top of the unsplit plan);
+// everything else with such tables runs on the LDS-table engine's global-gather variant.
+constexpr int64_t WIDE_MIN_ROWS = 512;
 struct WideQ {
     const uint32_t *qw;
     const uint32_t *qflags;
@@ -133,9 +133,9 @@ struct WideQ {
     int Jp, nchunks;
 };
 bool wide_shape_eligible(int64_t R, int batch);
-bool wide_eligible(int m, const GemmDesc &d);
-size_t wide_workspace_bytes(int64_t R, int64_t K, int batch);
-int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, hipStream_t stream);
+bool wide_eligible(int m, const GemmDesc &d, bool may_split);
+size_t wide_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch);
+int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, bool may_split, hipStream_t stream);
 // workspace that serves a dense problem with any table: the larger of gemm_workspace_bytes and
 // what the row-staged engine needs
 size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches);

@@ -157,7 +157,7 @@ def convam_filter_grad(lut, input, filter_sizes, out_backprop, strides=(1, 1), p
         raise ValueError("out_backprop / input do not match filter_sizes")
     out = torch.empty((kh, kw, c, oc), dtype=torch.float32, device=x.device)
     lib = load_library()
-    nbytes = lib.amsim_convam_filter_grad_workspace_bytes(n, oh, ow, oc, kh, kw, c)
+    nbytes = lib.amsim_convam_filter_grad_workspace_bytes_for(lut.handle, n, oh, ow, oc, kh, kw, c)
     ws, wsp = _workspace(nbytes, x.device)
     check(lib.amsim_convam_filter_grad_f32(lut.handle, _ptr(x), _ptr(dy), h, wd, n, c, ow, oh, oc, pl, pt,
                                            strides[0], strides[1], kw, kh, _ptr(out), wsp, nbytes, _stream()))

@@ -193,6 +193,11 @@ int amsim_convam_input_grad_f32(amsim_lut_t lut, const float *grad, int hole_gra
  * cuda_kernel.cu:431-461) */
 size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth,
                                                 int filter_rows, int filter_cols, int in_depth);
+/* The query for a given table: as amsim_convam_workspace_bytes_for, for the filter gradient (the
+ * transposed gather of the input that the row-staged engine reads, padded to 1024 rows, + the
+ * partial sums of its sliced reduction: about 4x faster than one global gather per product). */
+size_t amsim_convam_filter_grad_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols,
+                                                    int out_depth, int filter_rows, int filter_cols, int in_depth);
 int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const float *grad, int input_rows,
                                  int input_cols, int batch, int in_depth, int out_cols, int out_rows,
                                  int out_depth, int filter_left_offset, int filter_top_offset, int stride_rows,
