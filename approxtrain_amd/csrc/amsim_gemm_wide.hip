@@ -296,7 +296,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
             // dynamically (small code, one product at a time) while the fast path keeps them in
             // registers.
             const __attribute__((address_space(4))) QDesc &qd = *(const __attribute__((address_space(4))) QDesc *)(uintptr_t)a.qdesc;
-            const float *qsrc = qd.base;
+            const float *qsrc = qd.base + (int64_t)qb * qd.batch_stride;  // this batch item's operand
             float tmp[RPT * WIDE_TN];
             uint32_t praw[RPT];
 #pragma unroll

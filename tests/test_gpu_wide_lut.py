@@ -271,3 +271,65 @@ def test_row_staged_tile_heights(luts, M, N, K):
     A, B = _ops(rng, M, N, K, 0, 0)
     got = host(functors.gemm(lut, dev(A), dev(B)))
     assert np.array_equal(got.view(np.uint32), cpu.gemm(img, 11, A, B).view(np.uint32))
+
+
+SPECIALS = np.array([np.inf, -np.inf, np.nan, 1e-40, -1e-42, 3e38, -3e38, 1e-30, 2e-38, 0.0, -0.0], dtype=np.float32)
+
+
+def _spice(rng, a, p):
+    if p <= 0:
+        return a
+    hit = rng.random(a.shape) < p
+    a = a.copy()
+    a[hit] = rng.choice(SPECIALS, size=int(hit.sum()))
+    return a
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_on_wide_tables(luts, seed):
+    """Seeded sweep at shapes that reach the row-staged engine (512 or more rows over the lanes):
+    GEMMs with transposes and batches, and the three convolution passes, for widths 8..11; a third of
+    the cases carry special values (inf, NaN, subnormals, huge, tiny) in every operand.  Whole
+    reductions: bit-equal to the oracle (NaN as a class)."""
+    from approxtrain_amd import functors
+    rng = np.random.default_rng(4000 + seed)
+    m = int(rng.choice([8, 9, 10, 11]))
+    kind = str(rng.choice(["MBM", "MIT"]))
+    lut, img = luts(kind, m)
+    p = (0.0, 0.0, 0.003)[seed % 3]
+    if seed % 2 == 0:
+        big, small, K = int(rng.integers(512, 5000)), int(rng.integers(1, 40)), int(rng.integers(1, 150))
+        M, N = (big, small) if seed % 4 == 0 else (small, big)
+        nb = int(rng.choice([0, 0, 2]))
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        sa = ((nb,) if nb else ()) + ((K, M) if ta else (M, K))
+        sb = ((nb,) if nb else ()) + ((N, K) if tb else (K, N))
+        A = _spice(rng, rng.standard_normal(sa).astype(np.float32), p)
+        B = _spice(rng, rng.standard_normal(sb).astype(np.float32), p)
+        got = host(functors.gemm(lut, dev(A), dev(B), trans_a=ta, trans_b=tb))
+        if nb:
+            want = np.stack([cpu.gemm(img, m, A[i], B[i], transA=int(ta), transB=int(tb)) for i in range(nb)])
+        else:
+            want = cpu.gemm(img, m, A, B, transA=int(ta), transB=int(tb))
+        assert got.shape == want.shape and np.all(same_bits_or_both_nan(got, want)), (m, M, N, K, nb, ta, tb)
+    else:
+        c = int(rng.choice([3, 8, 24, 64, 70]))
+        oc = int(rng.choice([1, 5, 16, 24]))
+        kh, kw = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+        if kh * kw * c < 512 and seed % 4 == 1:
+            c = -(-512 // (kh * kw)) + int(rng.integers(0, 9))      # enough filter elements for the filter gradient's rows
+        n, h, w = int(rng.integers(1, 4)), int(rng.integers(kh + 8, kh + 30)), int(rng.integers(kw + 8, kw + 30))
+        st = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        padding = str(rng.choice(["SAME", "VALID"]))
+        xs, ws = (n, h, w, c), (kh, kw, c, oc)
+        x = _spice(rng, rng.standard_normal(xs).astype(np.float32) * (rng.random(xs) > 0.3), p)
+        wt = _spice(rng, rng.standard_normal(ws).astype(np.float32), p)
+        want_y = cpu.conv2d_fwd(img, m, x, wt, st, padding)
+        dy = _spice(rng, rng.standard_normal(want_y.shape).astype(np.float32), p)
+        got = [host(functors.convam(lut, dev(x), dev(wt), st, padding)),
+               host(functors.convam_input_grad(lut, xs, dev(wt), dev(dy), st, padding)),
+               host(functors.convam_filter_grad(lut, dev(x), ws, dev(dy), st, padding))]
+        want = [want_y, cpu.conv2d_grad_input(img, m, xs, wt, dy, st, padding),
+                cpu.conv2d_grad_filter(img, m, x, ws, dy, st, padding)]
+        for g, v in zip(got, want):
+            assert np.all(same_bits_or_both_nan(g, v)), (m, xs, ws, st, padding)
