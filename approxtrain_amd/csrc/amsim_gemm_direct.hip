@@ -116,9 +116,11 @@ __device__ __forceinline__ void step_walk(const PDesc &p, KWalk &w)
     }
 }
 
-// TN  columns per wavefront;  PK lane-operand source;  VEC4: dense source contiguous along the
-// reduction and 16-byte aligned, read four steps at a time
-template <int TN, int PK, bool VEC4>
+// TN  columns per wavefront;  PK lane-operand source;  VEC: reduction steps read per load (4 or 2 where
+// the source is contiguous along the reduction and aligned to as many floats: row-major dense
+// operands, and the channels of a patch source whose depth is a multiple of VEC -- one window test per
+// load instead of one per element)
+template <int TN, int PK, int VEC>
 __global__ __launch_bounds__(WG_THREADS, 4) void lutgemm_direct_kernel(DArgs a)
 {
     constexpr int SI = steps_per_iteration(TN);      // reduction steps per loop iteration
@@ -194,12 +196,36 @@ __global__ __launch_bounds__(WG_THREADS, 4) void lutgemm_direct_kernel(DArgs a)
             const uint32_t qk = (uint32_t)k0 + nb * KB + lane / TN, qj = (uint32_t)j0 + lane % TN;
             qraw[nb] = (live && lane < KB * TN && qk < (uint32_t)kend) ? q_raw_bits(a.q, qbase, (uint32_t)a.K, (uint32_t)a.J, qk, qj) : 0u;
         }
-        if (PK == P_DENSE && VEC4) {
+        if (PK == P_DENSE && VEC == 4) {
 #pragma unroll
             for (int kk = 0; kk < SI; kk += 4) {
                 uint4 q4 = make_uint4(0, 0, 0, 0);
                 if (live && row.valid && k0 + kk < kend) q4 = *reinterpret_cast<const uint4 *>(prow + k0 + kk);  // kend % 4 == 0 here
                 praw[kk] = q4.x; praw[kk + 1] = q4.y; praw[kk + 2] = q4.z; praw[kk + 3] = q4.w;
+            }
+        } else if (PK == P_PATCH && VEC > 1) {
+            // VEC channels of one window position per load: k0, the slice bounds and the depth are
+            // multiples of VEC, so a group never straddles a window position or the slice's end
+#pragma unroll
+            for (int kk = 0; kk < SI; kk += VEC) {
+                uint32_t v[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) v[i] = 0u;
+                if (live && row.valid && k0 + kk < kend && (unsigned)(row.vy0 + walk.a) < (unsigned)a.p.SH &&
+                    (unsigned)(row.vx0 + walk.b) < (unsigned)a.p.SW) {
+                    const float *src = pbase + row.base + (walk.a * a.p.SW + walk.b) * a.p.C + walk.c;
+                    if (VEC == 4) {
+                        const uint4 t = *reinterpret_cast<const uint4 *>(src);
+                        v[0] = t.x; v[1] = t.y; v[VEC - 2] = t.z; v[VEC - 1] = t.w;
+                    } else {
+                        const uint2 t = *reinterpret_cast<const uint2 *>(src);
+                        v[0] = t.x; v[1] = t.y;
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) praw[kk + i] = v[i];
+                walk.c += VEC;
+                if (walk.c == a.p.C) { walk.c = 0; if (++walk.b == a.p.KW) { walk.b = 0; ++walk.a; } }
             }
         } else {
 #pragma unroll
@@ -380,12 +406,16 @@ void launch_direct_tn(const DArgs &a, dim3 grid, hipStream_t stream)
     if (p.kind == P_DENSE) {
         const bool vec = p.sk == 1 && p.sr % 4 == 0 && p.batch_stride % 4 == 0 &&
                          a.K % 4 == 0 && aligned16(p.base);
-        if (vec) lutgemm_direct_kernel<TN, P_DENSE, true><<<grid, WG_THREADS, 0, stream>>>(a);
-        else lutgemm_direct_kernel<TN, P_DENSE, false><<<grid, WG_THREADS, 0, stream>>>(a);
+        if (vec) lutgemm_direct_kernel<TN, P_DENSE, 4><<<grid, WG_THREADS, 0, stream>>>(a);
+        else lutgemm_direct_kernel<TN, P_DENSE, 1><<<grid, WG_THREADS, 0, stream>>>(a);
     } else if (p.kind == P_PATCH) {
-        lutgemm_direct_kernel<TN, P_PATCH, false><<<grid, WG_THREADS, 0, stream>>>(a);
+        const bool even = p.C % 2 == 0 && p.batch_stride % 2 == 0 && ((uintptr_t)p.base & 7) == 0;
+        if (p.C % 4 == 0 && p.batch_stride % 4 == 0 && aligned16(p.base))
+            lutgemm_direct_kernel<TN, P_PATCH, 4><<<grid, WG_THREADS, 0, stream>>>(a);
+        else if (even) lutgemm_direct_kernel<TN, P_PATCH, 2><<<grid, WG_THREADS, 0, stream>>>(a);
+        else lutgemm_direct_kernel<TN, P_PATCH, 1><<<grid, WG_THREADS, 0, stream>>>(a);
     } else {
-        lutgemm_direct_kernel<TN, P_GF, false><<<grid, WG_THREADS, 0, stream>>>(a);
+        lutgemm_direct_kernel<TN, P_GF, 1><<<grid, WG_THREADS, 0, stream>>>(a);
     }
 }
 
