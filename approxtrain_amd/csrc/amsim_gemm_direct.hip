@@ -16,7 +16,7 @@
 //     in the workspace, summed by the fixed-order reduction kernel);
 //   * the byte-wide LUT image sits in LDS as in the main engine (all lanes of a gather inside one
 //     row: conflict-free).
-// Per product: two v_readlane, the address add, the byte -> factor step and the FMA -- about half
+// Per product: one v_readlane, the address add, the byte -> factor step and the FMA -- about half
 // the main engine's rate per instruction slot, which is irrelevant where launches and latencies
 // dominate: LeNet-sized layers (30-60 MMAC) run 15-50 % faster here than as pre-pass + main + reduction,
 // filter gradients of such layers (few outputs, long reduction) up to 2x.
@@ -244,48 +244,44 @@ __global__ __launch_bounds__(WG_THREADS, 4) void lutgemm_direct_kernel(DArgs a)
         if (!__any(unsafe)) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const uint32_t qtop = qraw[nb] & 0xff800000u;
-                // zero (and padding) elements select the all-zero LUT row that follows the table
-                const uint32_t qrow = ((qraw[nb] & 0x7fffffffu) ? ((qraw[nb] & 0x7fffffu) >> mshift) : (1u << m)) << m;
-                // The KB * TN products of this decode in groups of G: a group's row offsets come back as
-                // scalars (v_readlane), its addresses and gathers go out together, and while they are in
-                // flight the group before it is finished (exponent words, byte -> factor, FMA).  The
-                // fences keep the scheduler from serialising a group through one scalar register and from
-                // draining the LDS queue after every few gathers: a lone wavefront has nothing else to
-                // hide that latency with.
+                // sign|exponent in the top 9 bits, LUT row offset below: one register, read back once per product.
+                // Zero (and padding) elements select the all-zero LUT row that follows the table.
+                const uint32_t qword = (qraw[nb] & 0xff800000u) |
+                                       (((qraw[nb] & 0x7fffffffu) ? ((qraw[nb] & 0x7fffffu) >> mshift) : (1u << m)) << m);
+                // The KB * TN products of this decode in groups of G: a group's words come back as scalars
+                // (v_readlane), its addresses and gathers go out together, and while they are in flight the
+                // group before it is finished (byte -> factor, FMA).  The fences keep the scheduler from
+                // serialising a group through one scalar register and from draining the LDS queue after
+                // every few gathers: a lone wavefront has nothing else to hide that latency with.
                 constexpr int PAIRS = KB * TN;
                 constexpr int G = PAIRS < 8 ? PAIRS : 8;
-                uint32_t lb[2][G];
-                auto gather_group = [&](int g0, uint32_t (&dst)[G]) {
-                    uint32_t srow[G];
+                uint32_t lb[2][G], sw[2][G];
+                auto gather_group = [&](int g0, uint32_t (&dst)[G], uint32_t (&words)[G]) {
 #pragma unroll
-                    for (int g = 0; g < G; ++g) srow[g] = __builtin_amdgcn_readlane(qrow, g0 + g);
+                    for (int g = 0; g < G; ++g) words[g] = __builtin_amdgcn_readlane(qword, g0 + g);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int g = 0; g < G; ++g) {
                         const uint32_t pv = praw[nb * KB + (g0 + g) / TN];
-                        dst[g] = lut_s[__builtin_amdgcn_ubfe(pv, (uint32_t)mshift, (uint32_t)m) + srow[g]];
+                        dst[g] = lut_s[__builtin_amdgcn_ubfe(pv, (uint32_t)mshift, (uint32_t)m) + (words[g] & 0x7fffffu)];
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 };
-                auto finish_group = [&](int g0, const uint32_t (&src)[G]) {
-                    uint32_t stop[G];
-#pragma unroll
-                    for (int g = 0; g < G; ++g) stop[g] = __builtin_amdgcn_readlane(qtop, g0 + g);
-                    __builtin_amdgcn_sched_barrier(0);
+                auto finish_group = [&](int g0, const uint32_t (&src)[G], const uint32_t (&words)[G]) {
 #pragma unroll
                     for (int g = 0; g < G; ++g) {
                         const uint32_t pv = praw[nb * KB + (g0 + g) / TN];
                         // (LUT byte << 16) + sign|exponent bits of q  ==  q_pow2 * 1.mant * 2^carry, exactly
-                        acc[(g0 + g) % TN] = __builtin_fmaf(u2f(pv & 0xff800000u), u2f((src[g] << 16) + stop[g]), acc[(g0 + g) % TN]);
+                        acc[(g0 + g) % TN] = __builtin_fmaf(u2f(pv & 0xff800000u), u2f((src[g] << 16) + (words[g] & 0xff800000u)),
+                                                            acc[(g0 + g) % TN]);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 };
-                gather_group(0, lb[0]);
+                gather_group(0, lb[0], sw[0]);
 #pragma unroll
                 for (int g0 = 0; g0 < PAIRS; g0 += G) {
-                    if (g0 + G < PAIRS) gather_group(g0 + G, lb[((g0 / G) + 1) & 1]);
-                    finish_group(g0, lb[(g0 / G) & 1]);
+                    if (g0 + G < PAIRS) gather_group(g0 + G, lb[((g0 / G) + 1) & 1], sw[((g0 / G) + 1) & 1]);
+                    finish_group(g0, lb[(g0 / G) & 1], sw[(g0 / G) & 1]);
                 }
             }
         } else {
