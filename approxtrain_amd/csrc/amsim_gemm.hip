@@ -910,6 +910,7 @@ size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_ba
     for (int w = WAVES_PER_SIMD - 1; w <= WAVES_PER_SIMD; ++w)
         need = std::max(need, make_plan(R, J, K, batch, q_batches, true, w).total);
     if (direct_shape_eligible(R, J, K, batch, true)) need = std::max(need, direct_workspace_bytes(R, J, K, batch));
+    if (batch == 1 && R <= KLANES_MAX_ROWS && R * J <= KLANES_MAX_OUTPUTS && K >= KLANES_MIN_REDUCTION) need = std::max(need, klanes_workspace_bytes(R, J, K));
     return need;
 }
 
@@ -1023,6 +1024,9 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     if (need && (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need))
         return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
                                              std::to_string(need) + " bytes");
+    // small filter gradients whose reductions may be split: the reduction over the lanes
+    if (engine == AMSIM_ENGINE_AUTO && may_split && klanes_eligible(lut.m, d))
+        return run_gemm_klanes(lut, d, workspace, workspace_bytes, stream);
     if (use_direct) return run_gemm_direct(lut, d, may_split, workspace, workspace_bytes, stream);
     if (wide_eligible(lut.m, d, may_split)) {
         // tables too wide for the LDS: the row-staged engine, if the workspace also holds the

@@ -152,6 +152,16 @@ bool direct_eligible(int m, const GemmDesc &d, bool any_size);
 size_t direct_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch);
 int run_gemm_direct(const Lut &lut, const GemmDesc &d, bool may_split, void *workspace, size_t workspace_bytes, hipStream_t stream);
 
+// ---- filter gradients of small layers: the reduction over the lanes ----------------------------
+// At most KLANES_MAX_ROWS filter elements, a long reduction (pixels), tables that fit the LDS,
+// reductions that may be split: see amsim_gemm_klanes.hip.
+constexpr int64_t KLANES_MAX_ROWS = 32;
+constexpr int64_t KLANES_MAX_OUTPUTS = 4096;
+constexpr int64_t KLANES_MIN_REDUCTION = 2048;
+bool klanes_eligible(int m, const GemmDesc &d);
+size_t klanes_workspace_bytes(int64_t R, int64_t J, int64_t K);
+int run_gemm_klanes(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream);
+
 int launch_mul(const Lut &lut, const float *a, const float *b, float *out, size_t n, hipStream_t stream);
 
 // Strided grad-input runs one sub-problem per residue class of the input pixels, each over the
