@@ -38,6 +38,45 @@ struct SafeRange {
     __device__ __forceinline__ bool unsafe() const { return tmax >= (191u << 24) || tmin < (64u << 24) - 1u; }
 };
 
+// The quick test above is per operand.  Whether a PRODUCT can take the fast form depends on both
+// operands: sign | (ea + eb - 127 + carry) << 23 | mantissa is right whenever both are normal (or
+// zero) and ea + eb lies in [128, 380] -- e.g. gradients far below 2^-63 multiplied with weights
+// near 1.  A set of operands is therefore summarised as a "span" word:
+//   bit 31      some operand fails the quick test (zero, or exponent in [64, 190])
+//   bit 30      a subnormal, an infinity or a NaN is among them (also set, conservatively, for the
+//               smallest normal binade and for the largest: the carry of the LUT entry is added to
+//               an operand's exponent field, which must not run into 255): only the full-domain
+//               product will do
+//   bits 15..8  smallest biased exponent among the non-zero operands (may read one less for an
+//               exact power of two), 255 if all are zero
+//   bits 7..0   largest biased exponent, 0 if all are zero
+// and two spans are compatible if every product of their operands can take the fast form.
+constexpr uint32_t SPAN_QUICK_FAIL = 0x80000000u, SPAN_HARD = 0x40000000u;
+__device__ __forceinline__ uint32_t span_word(const SafeRange &r)
+{
+    const uint32_t emax = r.tmax >> 24;
+    const bool all_zero = r.tmin == 0xffffffffu && r.tmax == 0u;
+    const uint32_t emin = all_zero ? 255u : (r.tmin == 0xffffffffu ? emax : r.tmin >> 24);
+    const bool hard = !all_zero && (emin == 0u || emax >= 254u);
+    return (r.unsafe() ? SPAN_QUICK_FAIL : 0u) | (hard ? SPAN_HARD : 0u) | (emin << 8) | emax;
+}
+__device__ __forceinline__ bool spans_compatible(uint32_t a, uint32_t b)
+{
+    if ((a | b) & SPAN_HARD) return false;
+    const uint32_t lo = ((a >> 8) & 255u) + ((b >> 8) & 255u), hi = (a & 255u) + (b & 255u);
+    return lo >= 128u && hi <= 380u;
+}
+// union of the lanes' ranges, the same in every lane
+__device__ __forceinline__ SafeRange wave_union(SafeRange r)
+{
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        r.tmax = max(r.tmax, (uint32_t)__shfl_xor((int)r.tmax, d, 64));
+        r.tmin = min(r.tmin, (uint32_t)__shfl_xor((int)r.tmin, d, 64));
+    }
+    return r;
+}
+
 // 64-bit add of a vector register pair and a scalar register pair in one instruction (the
 // compiler's own choice for this sum is a multiply-add form that issues several times slower).
 __device__ __forceinline__ uint64_t add_u64_vs(uint64_t v, uint64_t s_uniform)

@@ -59,7 +59,7 @@ struct KArgs {
                              // by the pre-pass): flagged chunks read its raw bits from there.  Kept behind a pointer
                              // so that its fields are loaded inside the rare path only and cost the inner loop no
                              // scalar registers.
-    const uint32_t *qflags;  // [qb][Jp/16][nchunks]
+    const uint32_t *qflags;  // [qb][Jp/16][nchunks] operand spans
     int q_batches;
     int64_t R, J, K;
     int Jp, nchunks;
@@ -83,8 +83,8 @@ struct KArgs {
 // uniform-operand pre-pass
 // ---------------------------------------------------------------------------
 // One wavefront per (32-row chunk, 16-column tile): decodes the tile, writes it
-// in the tile-major layout the main kernel streams, and flags the tile-chunk
-// if it holds an operand the fast product path cannot take.  blockIdx.x runs over
+// in the tile-major layout the main kernel streams, and records the tile-chunk's
+// operand span (exponent range, special values: amsim_device.h).  blockIdx.x runs over
 // (chunk, group of four column tiles), blockIdx.y over the batch.
 __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
 {
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
     const bool k_fast = (a.q.kind == Q_DENSE && a.q.sk == 1 && a.q.sj != 1) || (a.q.kind == Q_FLIP);
     __shared__ uint32_t turn[WG_THREADS / 64][KC][QT + 1];
     const int w = threadIdx.x >> 6;
-    int unsafe = 0;
+    SafeRange range;
 #pragma unroll
     for (int i = 0; i < KC * QT / 64; ++i) {
         const int e = lane + 64 * i;
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
         if (k_fast) { kk = e % KC; jj = e / KC; }
         else { jj = e % QT; kk = e / QT; }
         const uint32_t raw = q_raw_bits(a.q, base, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)ch * KC + kk, (uint32_t)jt * QT + jj);
-        unsafe |= operand_unsafe(raw) ? 1 : 0;
+        range.add(raw);
         // zero (and padding) elements select the all-zero LUT row that follows the table:
         // their product term is then exactly +-0 without a test in the inner loop
         const uint32_t mant = (raw & 0x7fffffffu) ? ((raw & 0x7fffffu) >> (23 - a.m)) : (1u << a.m);
@@ -129,8 +129,9 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
             qw[e] = turn[w][e / QT][e % QT];
         }
     }
-    const int any = __any(unsafe);
-    if (lane == 0) a.qflags[((size_t)qb * ntiles + jt) * a.nchunks + ch] = (uint32_t)any;
+    // the tile-chunk's span: top bit = "an operand fails the quick test", below it the exponent range
+    const uint32_t span = span_word(wave_union(range));
+    if (lane == 0) a.qflags[((size_t)qb * ntiles + jt) * a.nchunks + ch] = span;
 }
 
 int launch_q_prepass(const QArgs &qa, int q_batches, hipStream_t stream)
@@ -539,9 +540,22 @@ void lutgemm_kernel(KArgs a)
         if (tid == 0) pflag[(ch & 1) ^ 1] = 0u;
         if (ch + 1 < ch_end) load_chunk(ch + 1);  // in flight during the MACs below
         if (!active) continue;
-        const uint32_t q_unsafe = qflags[ch];
+        const uint32_t q_span = qflags[ch];
         const size_t qoff = (size_t)ch * KC * QT;
-        if (!(p_unsafe | q_unsafe)) {
+        // Both operands pass the quick test: fast products.  Else a second look before the slow path:
+        // the exponent range of THIS wavefront's rows of the staged tile against the uniform operand's --
+        // tiny gradients times ordinary weights, say, are still fast products.
+        bool fast = !(p_unsafe | (q_span & SPAN_QUICK_FAIL));
+        if (!fast) {
+            SafeRange mine;
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                const uint4 p4 = Pt4[g * GS + lrow];
+                mine.add(p4.x); mine.add(p4.y); mine.add(p4.z); mine.add(p4.w);
+            }
+            fast = spans_compatible(span_word(wave_union(mine)), q_span);
+        }
+        if (fast) {
             cq1_t qrow = qw + qoff;
 #pragma unroll 1
             for (int g = 0; g < NG; ++g) {

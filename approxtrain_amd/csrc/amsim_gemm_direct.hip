@@ -236,12 +236,16 @@ __global__ __launch_bounds__(WG_THREADS, 4) void lutgemm_direct_kernel(DArgs a)
         }
     };
     auto compute = [&](int64_t k0, const uint32_t (&qraw)[NB], const uint32_t (&praw)[SI]) {
-        int unsafe = 0;
+        SafeRange qr, pr;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) unsafe |= operand_unsafe(qraw[nb]) ? 1 : 0;
+        for (int nb = 0; nb < NB; ++nb) qr.add(qraw[nb]);
 #pragma unroll
-        for (int kk = 0; kk < SI; ++kk) unsafe |= operand_unsafe(praw[kk]) ? 1 : 0;
-        if (!__any(unsafe)) {
+        for (int kk = 0; kk < SI; ++kk) pr.add(praw[kk]);
+        // every operand passes the quick test, or (second look) the two operands' exponent ranges over
+        // these steps are such that every product can still take the fast form
+        bool fast = !__any((qr.unsafe() || pr.unsafe()) ? 1 : 0);
+        if (!fast) fast = spans_compatible(span_word(wave_union(pr)), span_word(wave_union(qr)));
+        if (fast) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 // sign|exponent in the top 9 bits, LUT row offset below: one register, read back once per product.

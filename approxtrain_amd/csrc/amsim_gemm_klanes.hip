@@ -140,12 +140,16 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_klanes_kernel(KLArgs a)
         }
     };
     auto compute = [&](const uint32_t (&xr)[RB], const uint32_t (&dr)[JB]) {
-        SafeRange range;
+        SafeRange xrange, drange;
 #pragma unroll
-        for (int rr = 0; rr < RB; ++rr) range.add(xr[rr]);
+        for (int rr = 0; rr < RB; ++rr) xrange.add(xr[rr]);
 #pragma unroll
-        for (int jj = 0; jj < JB; ++jj) range.add(dr[jj]);
-        if (!__any(range.unsafe() ? 1 : 0)) {
+        for (int jj = 0; jj < JB; ++jj) drange.add(dr[jj]);
+        // every operand passes the quick test, or (second look) the exponent ranges of this pass's inputs
+        // and gradients are such that every product can still take the fast form
+        bool fast = !__any((xrange.unsafe() || drange.unsafe()) ? 1 : 0);
+        if (!fast) fast = spans_compatible(span_word(wave_union(xrange)), span_word(wave_union(drange)));
+        if (fast) {
             uint32_t dcol[JB], dse[JB];
 #pragma unroll
             for (int jj = 0; jj < JB; ++jj) {

@@ -47,7 +47,7 @@ struct PTArgs {
     int64_t R, K, Rp;
     int nchunks;
     uint32_t *pt;      // [batch][nchunks * KC][Rp] raw bits
-    uint32_t *pflags;  // [batch][nchunks][Rp / 64]
+    uint32_t *pflags;  // [batch][nchunks][Rp / 64] operand spans
 };
 
 // One workgroup per (64-row group, 32-deep chunk) and batch item (blockIdx.y): reads the tile along
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
     // lanes along k where the source is contiguous there: row-major dense operands, and patches
     // (channels run fastest in both the image and the reduction index)
     const bool k_fast = a.p.kind == P_PATCH || (a.p.kind == P_DENSE && a.p.sk == 1 && a.p.sr != 1);
-    int unsafe = 0;
+    SafeRange range;
 #pragma unroll
     for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
         const int e = tid + WG_THREADS * i;
@@ -75,17 +75,26 @@ __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
         else { rl = e % PT_ROWS; kk = e / PT_ROWS; }
         const int64_t r = g * PT_ROWS + rl, k = ch * KC + kk;
         const uint32_t raw = p_raw_bits(a.p, pbase, a.R, a.K, r, k);
-        unsafe |= operand_unsafe(raw) ? 1 : 0;
+        range.add(raw);
         tile[kk][rl] = raw;
     }
-    const int any = __syncthreads_or(unsafe);
+    // the tile's operand span: per wavefront by shuffles, across the four through LDS
+    __shared__ uint32_t wave_range[WG_THREADS / 64][2];
+    range = wave_union(range);
+    if ((tid & 63) == 0) { wave_range[tid >> 6][0] = range.tmax; wave_range[tid >> 6][1] = range.tmin; }
+    __syncthreads();
 #pragma unroll
     for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
         const int e = tid + WG_THREADS * i;
         const int rl = e % PT_ROWS, kk = e / PT_ROWS;
         pt[(size_t)(ch * KC + kk) * a.Rp + g * PT_ROWS + rl] = tile[kk][rl];
     }
-    if (tid == 0) a.pflags[((size_t)bz * a.nchunks + ch) * G + g] = (uint32_t)any;
+    if (tid == 0) {
+        SafeRange all;
+#pragma unroll
+        for (int w = 0; w < WG_THREADS / 64; ++w) { all.tmax = max(all.tmax, wave_range[w][0]); all.tmin = min(all.tmin, wave_range[w][1]); }
+        a.pflags[((size_t)bz * a.nchunks + ch) * G + g] = span_word(all);
+    }
 }
 
 // LDS byte address of a pointer into a __shared__ object
@@ -264,10 +273,10 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     // fast stages, whose registers the rare path's state cannot crowd.
     int tile_flagged = 0;
     for (int ch = ch_beg + tid; ch < ch_end; ch += WIDE_THREADS)
-        tile_flagged |= (int)a.qflags[qt_index * a.nchunks + ch];
+        tile_flagged |= (int)(a.qflags[qt_index * a.nchunks + ch] >> 31);
     for (int i = tid; i < (ch_end - ch_beg) * (TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
-        tile_flagged |= (int)pfl[(size_t)(ch_beg + i / (TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (TILE_ROWS / PT_ROWS) +
-                                 i % (TILE_ROWS / PT_ROWS)];
+        tile_flagged |= (int)(pfl[(size_t)(ch_beg + i / (TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (TILE_ROWS / PT_ROWS) +
+                                  i % (TILE_ROWS / PT_ROWS)] >> 31);
     tile_flagged = __syncthreads_or(tile_flagged);
 
     // one stage: the rows of stage k + 1 are fetched while stage k gathers from `cur`, and regrouped
@@ -335,8 +344,26 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         }
     } else {
         for (int ch = ch_beg; ch < ch_end; ++ch) {
-            const uint32_t pf = lane < TILE_ROWS / PT_ROWS ? pfl[(size_t)ch * G + (size_t)bx * (TILE_ROWS / PT_ROWS) + lane] : 0u;
-            const bool unsafe = (qfl[ch] != 0u) | (__any(pf != 0u) != 0);
+            // spans of the tile's 64-row groups (one per lane: TILE_ROWS / 64 <= 64), joined; the chunk is
+            // slow only if a quick test failed AND the joined span is not compatible with the uniform operand's
+            SafeRange join;
+            uint32_t quick = qfl[ch] & SPAN_QUICK_FAIL, hard = 0u;
+            if (lane < TILE_ROWS / PT_ROWS) {
+                const uint32_t pf = pfl[(size_t)ch * G + (size_t)bx * (TILE_ROWS / PT_ROWS) + lane];
+                quick |= pf & SPAN_QUICK_FAIL;
+                hard = pf & SPAN_HARD;
+                if ((pf & 0xffffu) != 0xff00u) {  // (not an all-zero group)
+                    join.tmax = (pf & 255u) << 24;
+                    join.tmin = ((pf >> 8) & 255u) << 24;
+                }
+            }
+            bool unsafe = __any(quick != 0u) != 0;
+            if (unsafe) {
+                join = wave_union(join);
+                const uint32_t emax = join.tmax >> 24, emin = join.tmin == 0xffffffffu ? 255u : join.tmin >> 24;
+                const uint32_t pspan = (__any(hard != 0u) ? SPAN_HARD : 0u) | (emin << 8) | emax;
+                unsafe = !spans_compatible(pspan, qfl[ch]);
+            }
             if (!unsafe) {
 #pragma unroll 1
                 for (int kk = 0; kk < KC; kk += 2) {

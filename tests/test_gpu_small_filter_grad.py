@@ -71,3 +71,24 @@ def test_random_small_filter_gradients(seed):
     dy = rng.standard_normal(y_shape).astype(np.float32) * (rng.random(y_shape) > 0.1)
     kind, m = [("MBM", 7), ("MIT", 7), ("MIT", 5), ("MBM", 1)][seed % 4]
     _check(kind, m, x, ws, dy, st, padding)
+
+
+@pytest.mark.parametrize("sx,sdy", [(0, -80), (-30, -70), (-90, -60), (40, 50), (110, 60)])
+def test_far_off_exponents(sx, sdy):
+    """Gradients (and inputs) scaled far outside the quick test's exponent interval: the pass still
+    takes the fast product form when the two exponent ranges allow it, the full-domain product when
+    products would under- or overflow; checked against the oracle at the usual tolerance."""
+    from approxtrain_amd import functors
+    rng = np.random.default_rng(abs(sx) + 3 * abs(sdy))
+    xs, ws = (64, 20, 20, 1), (5, 5, 1, 6)
+    x = (rng.standard_normal(xs) * 2.0 ** sx).astype(np.float32)
+    dy = (rng.standard_normal((64, 20, 20, 6)) * 2.0 ** sdy).astype(np.float32)
+    split, whole, L = _handles("MIT", 7)
+    want = cpu.conv2d_grad_filter(L, 7, x, ws, dy, (1, 1), "SAME", threads=cpu.max_threads()).astype(np.float64)
+    got = host(functors.convam_filter_grad(split, dev(x), ws, dev(dy), (1, 1), "SAME")).astype(np.float64)
+    exact = host(functors.convam_filter_grad(whole, dev(x), ws, dev(dy), (1, 1), "SAME"))
+    assert np.array_equal(exact.view(np.uint32), want.astype(np.float32).view(np.uint32))
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    scale = np.abs(want[np.isfinite(want)]).max() if np.isfinite(want).any() else 0.0
+    fin = np.isfinite(want)
+    assert np.all(np.abs(got - want)[fin] <= 2e-4 * scale + 1e-45)   # 6400 products per output, partial sums in another order

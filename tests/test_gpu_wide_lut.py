@@ -333,3 +333,19 @@ def test_random_shapes_on_wide_tables(luts, seed):
                 cpu.conv2d_grad_filter(img, m, x, ws, dy, st, padding)]
         for g, v in zip(got, want):
             assert np.all(same_bits_or_both_nan(g, v)), (m, xs, ws, st, padding)
+
+
+@pytest.mark.parametrize("sa,sb", [(-90, 0), (0, -100), (-70, -50), (-100, -40), (60, 30), (100, 30), (-126, 40)])
+def test_row_staged_gemm_far_off_exponents(luts, sa, sb):
+    """Operands scaled by 2^sa and 2^sb: far outside the quick test's exponent interval, yet most
+    pairs of ranges still allow the fast product form (tiny times ordinary); where the products
+    would under- or overflow the chunk takes the full-domain product.  Bit-equal either way."""
+    from approxtrain_amd import functors
+    lut, img = luts("MBM", 11)
+    rng = np.random.default_rng(abs(sa) * 7 + abs(sb))
+    A, B = _ops(rng, 1100, 24, 70, 0, 0)
+    A = (A * np.float32(2.0) ** sa).astype(np.float32)
+    B = (B * np.float32(2.0) ** sb).astype(np.float32)
+    got = host(functors.gemm(lut, dev(A), dev(B)))
+    want = cpu.gemm(img, 11, A, B)
+    assert np.all(same_bits_or_both_nan(got, want))
