@@ -66,14 +66,27 @@ __device__ __forceinline__ bool spans_compatible(uint32_t a, uint32_t b)
     const uint32_t lo = ((a >> 8) & 255u) + ((b >> 8) & 255u), hi = (a & 255u) + (b & 255u);
     return lo >= 128u && hi <= 380u;
 }
-// union of the lanes' ranges, the same in every lane
+// union of the lanes' ranges, the same in every lane: max / min over the wavefront by data-parallel
+// primitives (shifts inside rows of 16 lanes, then broadcasts of a row's last lane to the rows after
+// it; lanes without a source keep the identity), the totals read back from lane 63
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false));  // row_shr:1
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false));  // row_shr:2
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xe, false));  // row_shr:4
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xc, false));  // row_shr:8
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false));  // row_bcast:15
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false));  // row_bcast:31
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+#else
+    return v;
+#endif
+}
 __device__ __forceinline__ SafeRange wave_union(SafeRange r)
 {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-        r.tmax = max(r.tmax, (uint32_t)__shfl_xor((int)r.tmax, d, 64));
-        r.tmin = min(r.tmin, (uint32_t)__shfl_xor((int)r.tmin, d, 64));
-    }
+    r.tmax = wave_max_u32(r.tmax);
+    r.tmin = ~wave_max_u32(~r.tmin);  // min(x) == ~max(~x)
     return r;
 }
 
