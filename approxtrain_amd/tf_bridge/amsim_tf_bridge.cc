@@ -128,7 +128,9 @@ void ConvamFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const T *input_
                                              T * /*im2col*/, const int /*padding*/,
                                              approx_mul_lut<GPUDevice> &mul_lut)
 {
-    const size_t ws = amsim_convam_workspace_bytes(batch, out_rows, out_cols, out_depth, filter_rows, filter_cols, in_depth);
+    // (the table-aware queries: tables wider than 7 bits also get the staged operand their engine reads)
+    const size_t ws = amsim_convam_workspace_bytes_for(handle_of(mul_lut), batch, out_rows, out_cols, out_depth, filter_rows,
+                                                       filter_cols, in_depth);
     std::lock_guard<std::mutex> hold(g_lock);
     check(amsim_convam_f32(handle_of(mul_lut), input_data, output_data, batch, out_rows, out_cols, out_depth,
                            stride_cols, stride_rows, filter_left_offset, filter_top_offset, filter_rows, filter_cols,
@@ -156,12 +158,9 @@ void ConvamInputGradFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const 
                                                       approx_mul_lut<GPUDevice> &mul_lut)
 {
     // with strides the call is a set of undilated sub-problems: size the scratch so each may split its reduction
-    const size_t ws = (stride_rows > 1 || stride_cols > 1)
-                          ? amsim_convam_input_grad_strided_workspace_bytes(batch, input_rows, input_cols, in_depth,
-                                                                            filter_rows, filter_cols, out_depth,
-                                                                            stride_rows, stride_cols, pad_top, pad_left)
-                          : amsim_convam_input_grad_workspace_bytes(batch, input_rows, input_cols, in_depth,
-                                                                    filter_rows, filter_cols, out_depth);
+    const size_t ws = amsim_convam_input_grad_workspace_bytes_for(handle_of(mul_lut), batch, input_rows, input_cols,
+                                                                  in_depth, filter_rows, filter_cols, out_depth,
+                                                                  stride_rows, stride_cols, pad_top, pad_left);
     std::lock_guard<std::mutex> hold(g_lock);
     check(amsim_convam_input_grad_f32(handle_of(mul_lut), grad, hole_grad_width, hole_grad_height, pad_top, pad_left,
                                       filter, filter_rows, filter_cols, out_depth, stride_rows, stride_cols, batch,
@@ -189,8 +188,8 @@ void ConvamFilterGradFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const
                                                        const int filter_cols, const int filter_rows, T *output,
                                                        approx_mul_lut<GPUDevice> &mul_lut)
 {
-    const size_t ws = amsim_convam_filter_grad_workspace_bytes(batch, out_rows, out_cols, out_depth, filter_rows,
-                                                               filter_cols, in_depth);
+    const size_t ws = amsim_convam_filter_grad_workspace_bytes_for(handle_of(mul_lut), batch, out_rows, out_cols, out_depth,
+                                                                   filter_rows, filter_cols, in_depth);
     std::lock_guard<std::mutex> hold(g_lock);
     check(amsim_convam_filter_grad_f32(handle_of(mul_lut), input, grad, input_rows, input_cols, batch, in_depth,
                                        out_cols, out_rows, out_depth, filter_left_offset, filter_top_offset,
