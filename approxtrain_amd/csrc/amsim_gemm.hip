@@ -517,6 +517,14 @@ void lutgemm_kernel(KArgs a)
     const int lrow = wr * 64 + lane;
     const int mshift = 23 - m;
 
+    // Touching the next chunk's pre-decoded uniform operand (one lane per 128-byte line of this
+    // wavefront's 2 KB) a chunk ahead brings it into L2 when it streams from HBM (filter gradients,
+    // large GEMMs): the scalar loads of the inner loop are waited for every four rows, and a miss all
+    // the way to HBM there stalls the wavefront.  The loaded word is never used; its register stays
+    // reserved until the next trip's tile loads -- issued after it, returned after it -- have landed.
+    const uint32_t *q_touch_ptr = a.qw + qtile + (size_t)lane * 32;
+    uint32_t q_touch = 0;
+
     for (int ch = ch_begin; ch < ch_end; ++ch) {
         // The instruction arbiter favours a SIMD's oldest waves, so left alone the workgroups
         // that share a CU finish far apart and the last ones run on a mostly empty CU.  Wave
@@ -538,7 +546,12 @@ void lutgemm_kernel(KArgs a)
         __syncthreads();
         const uint32_t p_unsafe = __builtin_amdgcn_readfirstlane(pflag[ch & 1]);
         if (tid == 0) pflag[(ch & 1) ^ 1] = 0u;
-        if (ch + 1 < ch_end) load_chunk(ch + 1);  // in flight during the MACs below
+        asm volatile("" ::"v"(q_touch));
+        if (ch + 1 < ch_end) {
+            if (active && lane < KC * QT * 4 / 128)
+                asm volatile("global_load_dword %0, %1, off" : "=v"(q_touch) : "v"(q_touch_ptr + (size_t)(ch + 1) * KC * QT) : "memory");
+            load_chunk(ch + 1);  // in flight during the MACs below
+        }
         if (!active) continue;
         const uint32_t q_span = qflags[ch];
         const size_t qoff = (size_t)ch * KC * QT;
