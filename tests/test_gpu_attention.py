@@ -136,6 +136,33 @@ def test_attention_operand_order_with_asymmetric_lut():
         assert np.array_equal(_bits(gk[b]), _bits(np.ascontiguousarray(cpu.gemm(L, 3, q[b], gs, transA=True).T)))
 
 
+def test_attention_core_of_the_encoder_block_at_full_size():
+    """The attention core of the benchmark's encoder block -- 32 sequences x 8 heads of 256 positions,
+    64 features per head, MBM_7 -- in one library call per direction: for a sample of (sequence, head)
+    items both forward products and all four backward products against the oracle GEMM, bit for bit,
+    on the intermediates the library produced; every other item must at least be finite."""
+    from approxtrain_amd import functors
+    rng = np.random.default_rng(77)
+    L = lut32("MBM", 7)
+    b, h, s, d = 32, 8, 256, 64
+    q, k, v, go = (rng.standard_normal((b, h, s, d)).astype(np.float32) for _ in range(4))
+    divisor = math.sqrt(float(d))
+    out, w = functors.attention(MBM, dev(q), dev(k), dev(v), divisor)
+    gq, gk, gv = functors.attention_grad(MBM, dev(q), dev(k), dev(v), w, dev(go), divisor)
+    for t in (out, w, gq, gk, gv):
+        assert torch.isfinite(t).all()
+    out, w, gq, gk, gv = (host(t) for t in (out, w, gq, gk, gv))
+    for (i, j) in ((0, 0), (13, 5), (31, 7), (20, 2)):
+        x = (cpu.gemm(L, 7, q[i, j], k[i, j], transB=True) / np.float32(divisor)).astype(np.float32)
+        np.testing.assert_allclose(w[i, j], _softmax64(x), rtol=2e-6, atol=1e-30)
+        assert np.array_equal(_bits(out[i, j]), _bits(cpu.gemm(L, 7, w[i, j], v[i, j]))), f"out, item {i, j}"
+        assert np.array_equal(_bits(gv[i, j]), _bits(cpu.gemm(L, 7, w[i, j], go[i, j], transA=True))), f"d(v), item {i, j}"
+        gs = _softmax_grad_like_the_kernel(w[i, j], cpu.gemm(L, 7, go[i, j], v[i, j], transB=True), divisor)
+        assert np.array_equal(_bits(gq[i, j]), _bits(cpu.gemm(L, 7, gs, k[i, j]))), f"d(q), item {i, j}"
+        want_gk = np.ascontiguousarray(cpu.gemm(L, 7, q[i, j], gs, transA=True).T)
+        assert np.array_equal(_bits(gk[i, j]), _bits(want_gk)), f"d(k), item {i, j}"
+
+
 @pytest.mark.parametrize("mask_shape", [None, (2, 1, 1, 48), (48, 48), (2, 1, 48, 48), (2, 3, 48, 48), (1, 3, 1, 48)])
 def test_attention_layer_matches_the_composed_ops(mask_shape):
     """DotProductAttention (one library call per direction) against the same chain spelled with
