@@ -35,6 +35,14 @@ constexpr int DIRECT_WAVES = WG_THREADS / 64;
 // lone wavefront issues an instruction about every 8 cycles, so an iteration of 16 steps x 16
 // columns takes 5 us: 16-column tiles use 8 steps so that short reductions can be cut finer.
 constexpr int steps_per_iteration(int tn) { return tn >= 16 ? 8 : 16; }
+// ... and per decode of the uniform operand (one element per lane): as many whole steps as 64 lanes
+// hold, a divisor of the iteration (six-column tiles: 8 steps on 48 lanes)
+constexpr int steps_per_decode(int tn)
+{
+    int kb = 64 / tn < steps_per_iteration(tn) ? 64 / tn : steps_per_iteration(tn);
+    while (steps_per_iteration(tn) % kb) --kb;
+    return kb;
+}
 
 struct DArgs {
     PDesc p;
@@ -124,7 +132,7 @@ template <int TN, int PK, int VEC>
 __global__ __launch_bounds__(WG_THREADS, 4) void lutgemm_direct_kernel(DArgs a)
 {
     constexpr int SI = steps_per_iteration(TN);      // reduction steps per loop iteration
-    constexpr int KB = 64 / TN < SI ? 64 / TN : SI;  // steps whose uniform operands one decode (one register) covers
+    constexpr int KB = steps_per_decode(TN);         // steps whose uniform operands one decode (one register) covers
     constexpr int NB = SI / KB;                      // decodes per iteration
     __shared__ __align__(16) uint8_t lut_s[LUT_LDS_BYTES];
     static_assert(DIRECT_WAVES * 16 * 64 * sizeof(float) <= LUT_LDS_BYTES, "the partial sums reuse the LUT's LDS");
@@ -369,7 +377,8 @@ struct DPlan {
     size_t partial_bytes;
 };
 
-inline int tn_of(int64_t J) { return J >= 9 ? 16 : J >= 5 ? 8 : J >= 3 ? 4 : J >= 2 ? 2 : 1; }
+// (six columns: LeNet-5's first convolution has six output channels, its second six input channels)
+inline int tn_of(int64_t J) { return J >= 9 ? 16 : J >= 7 ? 8 : J >= 5 ? 6 : J >= 3 ? 4 : J >= 2 ? 2 : 1; }
 
 // How a problem is cut: tiles of 64 rows x TN columns, and the reduction into wks slices inside a
 // workgroup times nsplit across workgroups, aiming at a few wavefronts per SIMD with at least a
@@ -484,6 +493,7 @@ int run_gemm_direct(const Lut &lut, const GemmDesc &d, bool may_split, void *wor
     switch (pl.TN) {
     case 16: launch_direct_tn<16>(a, grid, stream); break;
     case 8: launch_direct_tn<8>(a, grid, stream); break;
+    case 6: launch_direct_tn<6>(a, grid, stream); break;
     case 4: launch_direct_tn<4>(a, grid, stream); break;
     case 2: launch_direct_tn<2>(a, grid, stream); break;
     default: launch_direct_tn<1>(a, grid, stream); break;
