@@ -11,11 +11,11 @@ fraction of the VALU-issue / LDS-gather roofline of the GEMM kernel's
 instruction mix (peaks measured on this device by micro-kernels in the same
 run, nominal figures beside them), the other benchmark configurations (dense
 layer, LeNet-5 convolutions, the 4096^3 GEMM sweep over ten tables, the
-attention block) under "configs", and the CPU oracle timed on a bounded sample
+attention block, and every convolution of ResNet-50's bottleneck stages) under "configs", and the CPU oracle timed on a bounded sample
 of the headline workload on the host cores.
 
 `--only NAME` runs one workload alone (headline, cfg1, cfg2, cfg4, cfg4-m11,
-cfg5) without micro-kernels or CPU baseline: the form the profiler runs.
+cfg5, resnet50) without micro-kernels or CPU baseline: the form the profiler runs.
 """
 import argparse
 import ctypes as C
@@ -323,6 +323,52 @@ def run_cfg5(roof):
     return out
 
 
+def run_resnet50(roof):
+    """Every convolution of ResNet-50's bottleneck stages 2-5 (the layout profile/resnet50.py:295-313
+    builds: per stage one block with a strided 1x1 and a 1x1 shortcut, then identity blocks of
+    1x1 -> 3x3 -> 1x1) at batch 32, MBM_7: forward, grad-input and grad-filter of each distinct layer
+    shape timed once and weighted by how often the model holds it.  Two sizes: feature maps 56 / 28 /
+    14 / 7 (an ImageNet-sized input behind the stem and pooling; its stage-2 3x3 layer is the headline
+    workload) and 32 / 16 / 8 / 4 on a 3-channel image (the reference's CIFAR-10 profile model)."""
+    import torch
+    from approxtrain_amd import functors
+    lut = make_lut("MBM", 7)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(20)
+    out = {}
+    for label, hw0, cin0 in (("feature_maps_56_to_7", 56, 64), ("feature_maps_32_to_4_cifar", 32, 3)):
+        layers = []  # (name, H = W, Cin, Cout, k, stride, how many)
+        hw, cin = hw0, cin0
+        for stage, (f1, f3, nblocks, stride) in enumerate(((64, 256, 3, 1), (128, 512, 4, 2), (256, 1024, 6, 2), (512, 2048, 3, 2)), start=2):
+            ohw = (hw - 1) // stride + 1
+            layers += [("s%da_1x1/%d_%d_%d" % (stage, stride, cin, f1), hw, cin, f1, 1, stride, 1),
+                       ("s%da_shortcut_1x1/%d_%d_%d" % (stage, stride, cin, f3), hw, cin, f3, 1, stride, 1),
+                       ("s%d_3x3_%d_%d" % (stage, f1, f1), ohw, f1, f1, 3, 1, nblocks),
+                       ("s%d_1x1_%d_%d" % (stage, f1, f3), ohw, f1, f3, 1, 1, nblocks),
+                       ("s%d_1x1_%d_%d" % (stage, f3, f1), ohw, f3, f1, 1, 1, nblocks - 1)]
+            hw, cin = ohw, f3
+        total_ms = total_macs = 0.0
+        per_layer = {}
+        for name, hw, cin, cout, k, stride, count in layers:
+            xs, ws, pad = (32, hw, hw, cin), (k, k, cin, cout), ("SAME" if k == 3 else "VALID")
+            x = torch.relu(torch.randn(*xs, device="cuda", generator=gen))
+            w = torch.randn(*ws, device="cuda", generator=gen) * math.sqrt(2.0 / (k * k * cin))
+            y = functors.convam(lut, x, w, (stride, stride), pad)
+            dy = torch.randn(*y.shape, device="cuda", generator=gen)
+            macs = y.numel() * k * k * cin
+            ms = [device_ms_graph(lambda: functors.convam(lut, x, w, (stride, stride), pad), calls=10, replays=3),
+                  device_ms_graph(lambda: functors.convam_input_grad(lut, xs, w, dy, (stride, stride), pad), calls=10, replays=3),
+                  device_ms_graph(lambda: functors.convam_filter_grad(lut, x, ws, dy, (stride, stride), pad), calls=10, replays=3)]
+            total_ms += sum(ms) * count
+            total_macs += 3.0 * macs * count
+            per_layer[name] = {"count": count, "mmacs_per_pass": round(macs / 1e6, 1),
+                               "fwd_gi_gf_gmacs": [round(macs / (t * 1e-3) / 1e9, 1) for t in ms]}
+        e = _entry(total_macs, total_ms, roof)
+        e["layers"] = per_layer
+        out[label] = e
+    return out
+
+
 def calibration_copy(lib):
     """One plain copy of known size (64 MiB read + 64 MiB written), outside every timed region:
     the kernel that FETCH_SIZE / WRITE_SIZE counter readings are scaled against."""
@@ -341,7 +387,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="headline workload only")
-    ap.add_argument("--only", default=None, help="run one workload alone: headline, cfg1, cfg2, cfg4, cfg4-m11, cfg5")
+    ap.add_argument("--only", default=None, help="run one workload alone: headline, cfg1, cfg2, cfg4, cfg4-m11, cfg5, resnet50")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -359,7 +405,8 @@ def main():
 
     if args.only and args.only != "headline":
         runners = {"cfg1": lambda: run_cfg1(None), "cfg2": lambda: run_cfg2(None), "cfg4": lambda: run_cfg4(None, None),
-                   "cfg4-m11": lambda: run_cfg4(None, None, tables={("MBM", 11), ("MIT", 11)}), "cfg5": lambda: run_cfg5(None)}
+                   "cfg4-m11": lambda: run_cfg4(None, None, tables={("MBM", 11), ("MIT", 11)}), "cfg5": lambda: run_cfg5(None),
+                   "resnet50": lambda: run_resnet50(None)}
         if args.only not in runners:
             sys.exit("unknown workload " + args.only)
         calibration_copy(lib)
@@ -475,6 +522,7 @@ def main():
                     "roofline.wide_table_bounds_gmacs -- bytes pulled in from L2 at 1.5 per product, the factor + FMA "
                     "instruction pair, scattered 16-byte LDS reads)",
             "cfg1": run_cfg1(peak), "cfg2": run_cfg2(peak), "cfg4": run_cfg4(peak, wide_peak), "cfg5": run_cfg5(peak),
+            "resnet50_convolutions_batch32": run_resnet50(peak),
         }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(x, w, dy)
