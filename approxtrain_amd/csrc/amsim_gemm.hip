@@ -179,23 +179,29 @@ __device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t 
 // main kernel
 // ---------------------------------------------------------------------------
 // TN     outputs per lane (uniform-dimension tile of one wave)
-// WR     row tiles per workgroup (waves are arranged WR x 4/WR)
+// WR     row tiles per workgroup (waves are arranged WR x 4/WR); 0: one row tile, one column group,
+//        the reduction rows of every chunk dealt out to the four waves (split reductions only)
 // PK     lane-operand source (PKind)
 // STAGE  how the staging threads walk the tile (STAGE_*)
 // LUTG   false: byte LUT image resident in LDS (mantissa width <= 7)
 //        true:  16-bit LUT image gathered from global memory through L2 / MALL
 //               (widths 8..11; a 2^22-entry table does not fit the 160 KB LDS)
+constexpr int WR_KSLICES = 0;  // value of WR that selects the reduction-slice arrangement
+
 template <int TN, int WR, int PK, int STAGE, bool LUTG>
-__global__ __launch_bounds__(WG_THREADS, (WR != 1 ? 2 : (PK == P_DENSE && STAGE != STAGE_K4) ? WAVES_PER_SIMD - 1 : WAVES_PER_SIMD))
+__global__ __launch_bounds__(WG_THREADS, (WR > 1 ? 2 : (PK == P_DENSE && STAGE != STAGE_K4) ? WAVES_PER_SIMD - 1 : WAVES_PER_SIMD))
 void lutgemm_kernel(KArgs a)
 {
-    constexpr int WC = 4 / WR;
-    constexpr int ROWS = 64 * WR;
+    // WR == 0 (WR_KSLICES): one row tile, one column group, and the four wavefronts take a quarter of
+    // every chunk's reduction rows each; their sums are added through LDS at the end, in wavefront order
+    constexpr bool KSLICES = WR == WR_KSLICES;
+    constexpr int WC = KSLICES ? 1 : 4 / (KSLICES ? 1 : WR);
+    constexpr int ROWS = KSLICES ? 64 : 64 * WR;
     constexpr int GS = ROWS + 1;  // padded group stride (in uint4): conflict-free transposing stores
     constexpr int ELEMS = ROWS * KC / WG_THREADS;
     constexpr int QUADS = ELEMS / 4;
 
-    __shared__ __align__(16) uint8_t lut_s[LUTG ? 16 : LUT_LDS_BYTES];
+    __shared__ __align__(16) uint8_t lut_s[LUTG ? (KSLICES ? 3 * TN * 64 * sizeof(float) : 16) : LUT_LDS_BYTES];
     const uint16_t *__restrict__ lut_g = reinterpret_cast<const uint16_t *>(a.lut_img);
     constexpr int ESHIFT = LUTG ? 8 : 16;  // LUT entry -> carry << 23 | mantissa
     __shared__ uint4 Pt4[NG * GS];
@@ -205,7 +211,8 @@ void lutgemm_kernel(KArgs a)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave / WC, wc = wave % WC;
+    const int wr = KSLICES ? 0 : wave / WC, wc = KSLICES ? 0 : wave % WC;
+    const int g_first = KSLICES ? wave * (NG / 4) : 0, g_last = KSLICES ? g_first + NG / 4 : NG;  // this wavefront's reduction-row groups of a chunk
     // Workgroups are handed to the 8 XCDs round-robin in launch order, and each
     // XCD has its own L2.  Renumber so that each XCD works on a contiguous run
     // of tiles (row tile fastest, then column group, then split / batch): the
@@ -569,9 +576,9 @@ void lutgemm_kernel(KArgs a)
             fast = spans_compatible(span_word(wave_union(mine)), q_span);
         }
         if (fast) {
-            cq1_t qrow = qw + qoff;
+            cq1_t qrow = qw + qoff + g_first * (KG * QT);
 #pragma unroll 1
-            for (int g = 0; g < NG; ++g) {
+            for (int g = g_first; g < g_last; ++g) {
                 // column pairs are unpacked with 64-bit scalar ops: half the SALU instructions
                 constexpr int TN2 = (TN + 1) / 2;
                 uint64_t qw2[KG][TN2];
@@ -622,7 +629,7 @@ void lutgemm_kernel(KArgs a)
             const __attribute__((address_space(4))) QDesc &qd = *(const __attribute__((address_space(4))) QDesc *)(uintptr_t)a.qdesc;
             const float *qsrc = qd.base + (int64_t)qb * qd.batch_stride;
 #pragma unroll 1
-            for (int kk = 0; kk < KC; ++kk) {
+            for (int kk = g_first * KG; kk < g_last * KG; ++kk) {
                 const uint32_t raw = Pt[((kk >> 2) * GS + lrow) * 4 + (kk & 3)];
                 const uint32_t ia = (raw & 0x7fffffu) >> mshift;
 #pragma unroll 1
@@ -640,7 +647,23 @@ void lutgemm_kernel(KArgs a)
     }
 
     const int64_t r = row0 + lrow;
-    if (!active) return;
+    if (!active) return;  // (with reduction slices `active` is the same for the whole workgroup)
+    if (KSLICES) {
+        // the four wavefronts' sums of one output, added in wavefront order through the LUT's LDS
+        float(*red)[TN][64] = reinterpret_cast<float(*)[TN][64]>(lut_s);
+        static_assert(LUTG || 3 * TN * 64 * sizeof(float) <= LUT_LDS_BYTES, "the slices' sums reuse the LUT's LDS");
+        __syncthreads();  // every wavefront is done gathering from the LUT
+        if (wave != 0) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) red[wave - 1][j][lane] = acc[j];
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int s = 0; s < 3; ++s)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[j] += red[s][j][lane];
+    }
     if (seg_nsplit == 1) {
         if (r < a.R) {
             float *o = a.out + (int64_t)bz * a.out_batch_stride + out_row_offset(a.ep.omap, r, a.so_r);
@@ -890,23 +913,52 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
     pl.WR = (jchunks >= 2 || R <= 64) ? 1 : 4;
     pl.Jp = (int)((J + QT - 1) / QT * QT);
     pl.nchunks = (int)((K + KC - 1) / KC);
-    const int rows = 64 * pl.WR, wc = 4 / pl.WR;
+
+    // the work shape of one wave arrangement, and what the cost model says it takes in seconds
+    struct Choice { Shape sh; double seconds; int rows; };
+    auto evaluate = [&](int WR) {
+        Choice c;
+        c.rows = WR > 1 ? 64 * WR : 64;
+        const int wc = WR == WR_KSLICES ? 1 : 4 / WR;
+        const int64_t Rp = (R + c.rows - 1) / c.rows * c.rows;
+        const int64_t rowtiles = Rp / c.rows;
+        const int64_t G = ((jchunks + wc - 1) / wc) * batch;
+        // resident workgroups: the 256-row kernels hold 53 KB of LDS and up to 170 VGPRs, three fit a CU
+        const int64_t slots = (int64_t)cus * (WR > 1 ? 3 : waves64);
+        c.sh.cps = pl.nchunks;
+        c.sh.main_rowtiles = rowtiles;
+        c.sh.tail_cps = pl.nchunks;
+        // one chunk of one workgroup on a full machine, and one pass over the output, in seconds
+        // (reduction slices: a quarter of the products per chunk behind the same staging and barriers -- a full
+        // machine of them takes 1.45 x the time per product; priced at 1.3, which picked best over a sweep of
+        // ResNet-50's layer shapes at small feature maps, the few-workgroup plans they compete with being
+        // underpriced by about as much)
+        const double chunk_s = (double)c.rows * (wc * pl.TN) * KC * slots / (MACS_PER_CU_S * cus) * (WR == WR_KSLICES ? 1.3 : 1.0);
+        if (split_k && pl.nchunks > 1) {
+            const double pass_s = 2.0 * (double)Rp * pl.Jp * batch * sizeof(float) / PARTIAL_BYTES_PER_S;
+            c.sh = shape_work(rowtiles, G, pl.nchunks, slots, true, pass_s / chunk_s);
+        } else {
+            c.sh.cost = pl.nchunks * occupancy_factor((double)(rowtiles * G) / slots);
+        }
+        const int64_t rounds = (rowtiles * G * c.sh.nsplit + slots - 1) / slots;
+        c.seconds = c.sh.cost * chunk_s + rounds * WORKGROUP_START_S;
+        return c;
+    };
+    Choice ch = evaluate(pl.WR);
+    // Few workgroups of the usual arrangement (half the slots or fewer) and a reduction that may be
+    // split: one column group per workgroup with the reduction rows dealt out to its four waves gives
+    // four times the workgroups and sums their slices inside the compute unit, without partial sums.
+    if (split_k && pl.nchunks > 1 && pl.TN == 16 && pl.WR == 1) {
+        const int64_t wgs = ((R + 63) / 64) * ((jchunks + 3) / 4) * batch;
+        if (2 * wgs <= (int64_t)cus * waves64) {
+            const Choice alt = evaluate(WR_KSLICES);
+            if (alt.seconds < 0.97 * ch.seconds) { ch = alt; pl.WR = WR_KSLICES; }
+        }
+    }
+    const Shape &sh = ch.sh;
+    const int rows = ch.rows;
     pl.Rp = (R + rows - 1) / rows * rows;
     const int64_t rowtiles = pl.Rp / rows;
-    const int64_t G = ((jchunks + wc - 1) / wc) * batch;
-    // resident workgroups: the 256-row kernels hold 53 KB of LDS and up to 170 VGPRs, three fit a CU
-    const int64_t slots = (int64_t)cus * (pl.WR == 1 ? waves64 : 3);
-
-    Shape sh;
-    sh.cps = pl.nchunks;
-    sh.main_rowtiles = rowtiles;
-    sh.tail_cps = pl.nchunks;
-    if (split_k && pl.nchunks > 1) {
-        // one chunk of one workgroup on a full machine, and one pass over the output, in seconds
-        const double chunk_s = (double)rows * (wc * pl.TN) * KC * slots / (MACS_PER_CU_S * cus);
-        const double pass_s = 2.0 * (double)pl.Rp * pl.Jp * batch * sizeof(float) / PARTIAL_BYTES_PER_S;
-        sh = shape_work(rowtiles, G, pl.nchunks, slots, true, pass_s / chunk_s);
-    }
     pl.nsplit = sh.nsplit;
     pl.chunks_per_split = sh.cps;
     pl.rows_main = sh.main_rowtiles == rowtiles ? R : sh.main_rowtiles * rows;
@@ -1011,6 +1063,7 @@ static void launch_tn(int TN, int WR, const KArgs &k, dim3 grid, hipStream_t str
     switch (TN) {
     case 16:
         if (WR == 1) launch_variant<16, 1, LUTG>(k, grid, stream);
+        else if (WR == WR_KSLICES) launch_variant<16, WR_KSLICES, LUTG>(k, grid, stream);
         else launch_variant<16, 4, LUTG>(k, grid, stream);
         break;
     case 8: launch_variant<8, 4, LUTG>(k, grid, stream); break;
@@ -1099,7 +1152,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.ep = Epilogue{d.bias_j, d.bias_r, d.act, d.omap};
     ka.vec_store = (d.so_j == 1 && d.so_r % 4 == 0 && d.out_batch_stride % 4 == 0 && aligned16(d.out)) ? 1 : 0;
 
-    const int rows = 64 * pl.WR, wc = 4 / pl.WR;
+    const int rows = pl.WR > 1 ? 64 * pl.WR : 64, wc = pl.WR == WR_KSLICES ? 1 : 4 / pl.WR;
     const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;
     const int64_t gy = (jchunks + wc - 1) / wc;
 

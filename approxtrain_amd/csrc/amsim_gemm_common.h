@@ -19,6 +19,7 @@ constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels ar
 constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
 constexpr double MACS_PER_CU_S = 13.0e12 / 256;  // planner's price of a MAC: what one compute unit sustains
 constexpr double PARTIAL_BYTES_PER_S = 3.0e12;   // planner's price of writing + re-reading partial sums
+constexpr double WORKGROUP_START_S = 3.5e-6;     // planner's price of a round of workgroup starts (LUT staging, first loads)
 
 
 typedef const __attribute__((address_space(4))) uint32_t *cq1_t;

@@ -253,9 +253,12 @@ def _plan(M, N, K, batch=1, ta=0, tb=0):
     (6272, 256, 2304, "split+tail"),
     (512, 512, 8192, "split"),          # few outputs, long reduction
     (51200, 64, 128, "whole"),          # short reduction: nothing to gain from splitting
-    (40, 6, 50000, "split"),            # one row tile
+    (40, 6, 50000, "slices+split"),     # one row tile: all four waves on its one column group
     (200704, 1, 150, "tail"),           # 256-row workgroups (one narrow column group): 768 slots + a split tail
     (50176, 6, 400, "split"),           # 256-row workgroups, reduction split three ways
+    (2048, 1024, 256, "slices+tail"),   # few row tiles, short reduction: its rows dealt out to a workgroup's four waves
+    (2048, 256, 1024, "slices+split"),  # ... and split across workgroups as well
+    (8192, 128, 256, "slices"),
 ])
 def test_planner_paths_match_the_oracle(amd, M, N, K, expect):
     """The work-shaping decisions (reduction split, tail rows split further, both with partial sums)
@@ -263,8 +266,10 @@ def test_planner_paths_match_the_oracle(amd, M, N, K, expect):
     from approxtrain_amd import ApproxMulLut
     p = _plan(M, N, K)
     split, tail = p["nsplit"] > 1, p["tail_nsplit"] > 0
+    assert (p["WR"] == 0) == expect.startswith("slices"), p
     assert {"tail": (not split) and tail, "split+tail": split and tail, "split": split and not tail,
-            "whole": (not split) and (not tail)}[expect], p
+            "whole": (not split) and (not tail), "slices": (not split) and (not tail), "slices+split": split and not tail,
+            "slices+tail": (not split) and tail}[expect], p
     _set_split(1)
     rng = np.random.default_rng(M + N + K)
     # a sample of the rows keeps the oracle fast: the GPU computes everything, rows are independent
