@@ -730,14 +730,28 @@ __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
     }
 }
 
-// Empty reduction: every output is the epilogue of zero (zeros without one).
+// Empty reduction: every output is the epilogue of zero (zeros without one).  VEC = 4: a thread
+// writes four consecutive columns of a row as one 16-byte store (rows contiguous, 16-byte aligned,
+// a multiple of four columns): the pixel classes of a strided grad-input that no filter tap
+// reaches are most of that tensor.
+template <int VEC>
 __global__ __launch_bounds__(WG_THREADS) void fill_empty_kernel(RArgs a)
 {
     const int64_t idx = (int64_t)blockIdx.x * WG_THREADS + threadIdx.x;
-    if (idx >= a.R * a.J) return;
-    const int64_t r = idx / a.J, j = idx - r * a.J;
-    a.out[(int64_t)blockIdx.y * a.out_batch_stride + out_row_offset(a.ep.omap, a.row_base + r, a.so_r) + j * a.so_j] =
-        apply_epilogue(a.ep, 0.0f, a.row_base + r, j);
+    const int64_t per_row = a.J / VEC;
+    if (idx >= a.R * per_row) return;
+    const int64_t r = idx / per_row, j = (idx - r * per_row) * VEC;
+    float *o = a.out + (int64_t)blockIdx.y * a.out_batch_stride + out_row_offset(a.ep.omap, a.row_base + r, a.so_r) + j * a.so_j;
+    if (VEC == 4) {
+        float4 v;
+        v.x = apply_epilogue(a.ep, 0.0f, a.row_base + r, j);
+        v.y = apply_epilogue(a.ep, 0.0f, a.row_base + r, j + 1);
+        v.z = apply_epilogue(a.ep, 0.0f, a.row_base + r, j + 2);
+        v.w = apply_epilogue(a.ep, 0.0f, a.row_base + r, j + 3);
+        *reinterpret_cast<float4 *>(o) = v;
+    } else {
+        *o = apply_epilogue(a.ep, 0.0f, a.row_base + r, j);
+    }
 }
 
 struct PoisonArgs {
@@ -1085,8 +1099,12 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0,
                  Epilogue{d.bias_j, d.bias_r, d.act, d.omap}};
         if (d.batch > 65535) return fail(AMSIM_ERR_UNSUPPORTED, "batch exceeds the grid limit");
-        fill_empty_kernel<<<dim3((unsigned)((d.R * d.J + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch), WG_THREADS, 0,
-                            stream>>>(ra);
+        const bool vec = d.J % 4 == 0 && d.so_j == 1 && d.so_r % 4 == 0 && d.out_batch_stride % 4 == 0 && aligned16(d.out);
+        const int64_t threads = d.R * (vec ? d.J / 4 : d.J);
+        if ((threads + WG_THREADS - 1) / WG_THREADS >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "output exceeds the grid limit");
+        const dim3 grid((unsigned)((threads + WG_THREADS - 1) / WG_THREADS), (unsigned)d.batch);
+        if (vec) fill_empty_kernel<4><<<grid, WG_THREADS, 0, stream>>>(ra);
+        else fill_empty_kernel<1><<<grid, WG_THREADS, 0, stream>>>(ra);
         AMSIM_HIP_CHECK(hipGetLastError());
         return AMSIM_OK;
     }
