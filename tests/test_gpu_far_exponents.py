@@ -37,6 +37,30 @@ def test_gemm(sa, sb, shape):
     assert np.all(same_bits_or_both_nan(got, cpu.gemm(L, 7, A, B)))
 
 
+@pytest.mark.parametrize("sa,sb", [(0, 0), (0, -80), (-85, 0), (-60, -60), (-70, -57), (-100, -30), (40, 40)])
+def test_gemm_with_split_reductions(sa, sb, amsim_engine):
+    """One row tile, three column groups, a long reduction, reductions free to be split: under the
+    LDS-table engine the reduction rows of every chunk are dealt out to a workgroup's four wavefronts
+    (and the chunks to many workgroups), so the second look and the full-domain products run inside
+    that arrangement too.  Within 1e-5 * sum|products| of the oracle's sequential chain."""
+    import ctypes as C
+    import approxtrain_amd
+    from approxtrain_amd import ApproxMulLut, functors
+    from tests.gpu_util import assert_close_sum_abs
+    lib = approxtrain_amd.load_library()
+    M, N, K = 64, 40, 2000
+    if amsim_engine == "lds_table":
+        info = (C.c_int64 * 8)()
+        assert lib.amsim_gemm_plan_info(0, 0, M, N, K, 1, info) == 0
+        assert info[1] == 0, list(info)  # the reduction-slice arrangement
+    lut, L = ApproxMulLut(lut_path("MBM", 7)), lut32("MBM", 7)
+    rng = np.random.default_rng(abs(sa) + 7 * abs(sb))
+    A = (rng.standard_normal((M, K)) * 2.0 ** sa).astype(np.float32) * (rng.random((M, K)) > 0.1)
+    B = (rng.standard_normal((K, N)) * 2.0 ** sb).astype(np.float32)
+    got = host(functors.gemm(lut, dev(A), dev(B)))
+    assert_close_sum_abs(got, cpu.gemm(L, 7, A, B), cpu.gemm_abs(L, 7, A, B), 1e-5)
+
+
 @pytest.mark.parametrize("sx,sw,sdy", [(0, 0, -80), (0, -10, -100), (-40, -50, -30), (30, 40, 50), (0, 0, 100)])
 def test_convolution_passes(sx, sw, sdy):
     from approxtrain_amd import functors
