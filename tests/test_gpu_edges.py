@@ -134,6 +134,46 @@ def test_runs_on_a_non_default_stream():
     assert np.array_equal(host(out).view(np.uint32), cpu.gemm(lut32("MBM", 7), 7, A, B).view(np.uint32))
 
 
+def test_two_host_threads_on_two_streams_with_their_own_handles():
+    """Calls are re-entrant: two host threads, each with its own stream, LUT handle (one keeps
+    reductions whole, the other lets them be split) and workspaces, interleave convolution and GEMM
+    calls; every result equals the one the same call gives alone."""
+    from concurrent.futures import ThreadPoolExecutor
+    import approxtrain_amd
+    from approxtrain_amd import ApproxMulLut, functors
+    lib = approxtrain_amd.load_library()
+    rng = np.random.default_rng(21)
+    xs, ws = (4, 20, 20, 16), (3, 3, 16, 24)
+    x, w = dev(rng.standard_normal(xs).astype(np.float32)), dev(rng.standard_normal(ws).astype(np.float32))
+    dy = dev(rng.standard_normal((4, 20, 20, 24)).astype(np.float32))
+    A, B = dev(rng.standard_normal((300, 700)).astype(np.float32)), dev(rng.standard_normal((700, 90)).astype(np.float32))
+    luts = [ApproxMulLut(lut_path("MBM", 7)), ApproxMulLut(lut_path("MIT", 7))]
+    assert lib.amsim_lut_set_split_k(luts[0].handle, 0) == 0 and lib.amsim_lut_set_split_k(luts[1].handle, 1) == 0
+
+    def calls(lut):
+        return [functors.convam(lut, x, w, (1, 1), "SAME"), functors.convam_input_grad(lut, xs, w, dy, (1, 1), "SAME"),
+                functors.convam_filter_grad(lut, x, ws, dy, (1, 1), "SAME"), functors.gemm(lut, A, B),
+                functors.gemm(lut, A, A, trans_b=True)]
+
+    alone = [[host(t) for t in calls(lut)] for lut in luts]
+    torch.cuda.synchronize()
+
+    def worker(i):
+        s = torch.cuda.Stream()
+        outs = []
+        with torch.cuda.stream(s):
+            for _ in range(8):
+                outs = calls(luts[i])
+        s.synchronize()
+        return [host(t) for t in outs]
+
+    with ThreadPoolExecutor(max_workers=2) as pool:
+        together = list(pool.map(worker, (0, 1)))
+    for i in range(2):
+        for got, want in zip(together[i], alone[i]):
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("xs,ws,stride,padding", [((2, 9, 8, 16), (1, 1, 16, 24), 2, "SAME"),     # taps reach 1 pixel in 4
                                                    ((2, 11, 7, 4), (2, 2, 4, 6), 3, "VALID"),      # filter smaller than stride
                                                    ((1, 12, 12, 32), (3, 3, 32, 32), 2, "SAME"),
