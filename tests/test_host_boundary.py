@@ -181,6 +181,35 @@ def test_workspace_queries_need_no_device():
     assert lib.amsim_matmulam_workspace_bytes(2, 3, 4, 5, 5, 6) == 0  # incompatible batches
 
 
+def test_planner_invariants_over_random_shapes():
+    """The work-shaping plan of the LDS-table engine (host code, no device needed): over random
+    problem shapes the reduction slices of the main part and of the tail cover every chunk with no
+    empty slice, a tail leaves whole tiles to the main part, and the arrangement that deals a
+    chunk's rows out to the four wavefronts is only used with 16-column tiles."""
+    import random
+    lib = approxtrain_amd.load_library()
+    info = (C.c_int64 * 8)()
+    rnd = random.Random(3)
+    slices = 0
+    for _ in range(30000):
+        M = rnd.choice([rnd.randint(1, 300), rnd.randint(1, 70000), rnd.randint(1, 300000)])
+        N = rnd.choice([rnd.randint(1, 20), rnd.randint(1, 600), rnd.randint(1, 5000)])
+        K = rnd.choice([rnd.randint(1, 100), rnd.randint(1, 5000), rnd.randint(1, 200000)])
+        batch = rnd.choice([1, 1, 1, 2, 7, 256])
+        assert lib.amsim_gemm_plan_info(0, 0, M, N, K, batch, info) == 0
+        TN, WR, nsplit, cps, rows_main, tail_nsplit, tail_cps, chunks = list(info)
+        shape = (M, N, K, batch, list(info))
+        assert TN in (1, 2, 4, 8, 16) and WR in (0, 1, 4), shape
+        assert nsplit >= 1 and cps >= 1 and nsplit * cps >= chunks > (nsplit - 1) * cps, shape
+        if tail_nsplit:
+            assert tail_nsplit * tail_cps >= chunks > (tail_nsplit - 1) * tail_cps, shape
+            assert rows_main > 0 and rows_main % (64 * max(WR, 1)) == 0, shape
+        if WR == 0:
+            slices += 1
+            assert TN == 16, shape
+    assert slices > 0
+
+
 def test_functors_refuse_host_tensors():
     from approxtrain_amd import functors
     with pytest.raises(TypeError, match="device memory"):
