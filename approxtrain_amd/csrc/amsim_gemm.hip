@@ -106,13 +106,25 @@ __global__ __launch_bounds__(WG_THREADS) void q_prepass_kernel(QArgs a)
     __shared__ uint32_t turn[WG_THREADS / 64][KC][QT + 1];
     const int w = threadIdx.x >> 6;
     SafeRange range;
+    // all of a lane's elements are fetched before the first is decoded and stored: the stores cannot be
+    // proven not to alias the source, so loads left between them would wait for one another
+    constexpr int PER_LANE = KC * QT / 64;
+    uint32_t raws[PER_LANE];
 #pragma unroll
-    for (int i = 0; i < KC * QT / 64; ++i) {
+    for (int i = 0; i < PER_LANE; ++i) {
         const int e = lane + 64 * i;
         int kk, jj;
         if (k_fast) { kk = e % KC; jj = e / KC; }
         else { jj = e % QT; kk = e / QT; }
-        const uint32_t raw = q_raw_bits(a.q, base, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)ch * KC + kk, (uint32_t)jt * QT + jj);
+        raws[i] = q_raw_bits(a.q, base, (uint32_t)a.K, (uint32_t)a.J, (uint32_t)ch * KC + kk, (uint32_t)jt * QT + jj);
+    }
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) {
+        const int e = lane + 64 * i;
+        int kk, jj;
+        if (k_fast) { kk = e % KC; jj = e / KC; }
+        else { jj = e % QT; kk = e / QT; }
+        const uint32_t raw = raws[i];
         range.add(raw);
         // zero (and padding) elements select the all-zero LUT row that follows the table:
         // their product term is then exactly +-0 without a test in the inner loop
