@@ -170,15 +170,17 @@ __device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t 
         int4 v = make_int4(0, -(1 << 28), 0, 0);
         if (r < R) {
             if (p.kind == P_PATCH) {
-                const int x = (int)(r % p.GW);
-                const int64_t t = r / p.GW;
-                const int y = (int)(t % p.GH);
-                const int b = (int)(t / p.GH);
+                // (row counts stay below 2^31: 32-bit divisions, a fraction of the 64-bit ones' instructions)
+                const uint32_t r32 = (uint32_t)r, gw = (uint32_t)p.GW, gh = (uint32_t)p.GH;
+                const int x = (int)(r32 % gw);
+                const uint32_t t = r32 / gw;
+                const int y = (int)(t % gh);
+                const int b = (int)(t / gh);
                 const int vy0 = y * p.sy - p.pt, vx0 = x * p.sx - p.pl;
                 v = make_int4(b * p.SH * p.SW * p.C, vy0, vx0, (b * p.SH * p.SW + vy0 * p.SW + vx0) * p.C);
             } else if (p.kind == P_GF) {
-                const int c = (int)(r % p.C);
-                const int t = (int)(r / p.C);
+                const int c = (int)((uint32_t)r % (uint32_t)p.C);
+                const int t = (int)((uint32_t)r / (uint32_t)p.C);
                 const int fx = t % p.KW, fy = t / p.KW;
                 v = make_int4((fy * p.SW + fx) * p.C + c, fy, fx, 0);
             }
@@ -321,9 +323,9 @@ void lutgemm_kernel(KArgs a)
     int cb_c = 0, cb_fx = 0, cb_fy = 0;
     const bool patch_walk = PK == P_PATCH && a.p.C >= KC;
     if (patch_walk) {
-        const int64_t kb = (int64_t)(split * seg_cps) * KC;
-        cb_c = (int)(kb % a.p.C);
-        const int t = (int)(kb / a.p.C);
+        const uint32_t kb = (uint32_t)(split * seg_cps) * KC;
+        cb_c = (int)(kb % (uint32_t)a.p.C);
+        const int t = (int)(kb / (uint32_t)a.p.C);
         cb_fx = t % a.p.KW;
         cb_fy = t / a.p.KW;
     }
@@ -332,8 +334,9 @@ void lutgemm_kernel(KArgs a)
             c = cb_c + koff; fx = cb_fx; fy = cb_fy;
             if (c >= a.p.C) { c -= a.p.C; if (++fx == a.p.KW) { fx = 0; ++fy; } }
         } else {
-            c = (int)(k % a.p.C);
-            const int t = (int)(k / a.p.C);
+            const uint32_t k32 = (uint32_t)k, c32 = (uint32_t)a.p.C;  // (k < 2^31)
+            c = (int)(k32 % c32);
+            const int t = (int)(k32 / c32);
             fx = t % a.p.KW; fy = t / a.p.KW;
         }
     };
@@ -353,8 +356,8 @@ void lutgemm_kernel(KArgs a)
     const bool gf_uniform = PK == P_GF && (a.p.C % ROWS == 0) && row0 + ROWS <= a.R;
     int gf_fy = 0, gf_fx = 0, gf_c0 = 0;
     if (gf_uniform) {
-        gf_c0 = (int)(row0 % a.p.C);
-        const int t = (int)(row0 / a.p.C);
+        gf_c0 = (int)((uint32_t)row0 % (uint32_t)a.p.C);
+        const int t = (int)((uint32_t)row0 / (uint32_t)a.p.C);
         gf_fx = t % a.p.KW;
         gf_fy = t / a.p.KW;
     }
@@ -426,10 +429,12 @@ void lutgemm_kernel(KArgs a)
             const int4 ri = rowinfo[rl];
             // the first pixel of this wave's run, decomposed once (wave-uniform), then walked
             const int64_t kfirst = k0 + __builtin_amdgcn_readfirstlane(tid / ROWS) * ELEMS;
-            int x = (int)(kfirst % a.p.GW);
-            const int64_t t = kfirst / a.p.GW;
-            int y = (int)(t % a.p.GH);
-            int b = (int)(t / a.p.GH);
+            // (the reduction is shorter than 2^31: 32-bit divisions, a fraction of the 64-bit ones' instructions)
+            const uint32_t kf32 = (uint32_t)kfirst, gw32 = (uint32_t)a.p.GW, gh32 = (uint32_t)a.p.GH;
+            int x = (int)(kf32 % gw32);
+            const uint32_t t = kf32 / gw32;
+            int y = (int)(t % gh32);
+            int b = (int)(t / gh32);
             if (gf_uniform) {
                 // all rows of the tile share (fy, fx): the pixel walk, the window test and the
                 // pixel's source offset are wave-uniform and stay in scalar registers; a lane
@@ -1106,6 +1111,8 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     if ((lut.m <= 7 && lut.img_ab == nullptr) || (lut.m > 7 && lut.img16_ab == nullptr))
         return fail(AMSIM_ERR_UNSUPPORTED, "LUT handle holds no device image for the GEMM path");
     if (const int rc = check_lut_device(lut)) return rc;
+    if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
+        return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
     if (d.K == 0) {
         // empty reduction: the output is all zeros (matmulam.cc:154-160)
         RArgs ra{nullptr, d.out, d.R, d.J, 0, d.so_r, d.so_j, d.out_batch_stride, 0, 0, d.batch, 0,
@@ -1120,8 +1127,6 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         AMSIM_HIP_CHECK(hipGetLastError());
         return AMSIM_OK;
     }
-    if (d.R >= (1ll << 31) || d.K >= (1ll << 31) || d.J >= (1ll << 24))
-        return fail(AMSIM_ERR_UNSUPPORTED, "GEMM extent too large");
     const int engine = lut.engine >= 0 ? lut.engine : g_engine.load();  // the handle's own setting wins
     const bool use_direct = engine != AMSIM_ENGINE_LDS_TABLE && direct_eligible(lut.m, d, engine == AMSIM_ENGINE_DIRECT);
     // the handle's own setting wins over the process default (read once per call)

@@ -37,10 +37,12 @@ struct Epilogue {
 __device__ __forceinline__ int64_t out_row_offset(const OutMap &m, int64_t r, int64_t so_r)
 {
     if (!m.enabled) return r * so_r;
-    const int x = (int)(r % m.GW);
-    const int64_t t = r / m.GW;
-    const int y = (int)(t % m.GH);
-    const int64_t b = t / m.GH;
+    // (mapped outputs have fewer than 2^31 rows: 32-bit divisions)
+    const uint32_t r32 = (uint32_t)r;
+    const int x = (int)(r32 % (uint32_t)m.GW);
+    const uint32_t t = r32 / (uint32_t)m.GW;
+    const int y = (int)(t % (uint32_t)m.GH);
+    const int64_t b = t / (uint32_t)m.GH;
     return ((b * m.H + (y * m.sy + m.oy)) * m.W + (x * m.sx + m.ox)) * so_r;
 }
 __device__ __forceinline__ float apply_epilogue(const Epilogue &e, float v, int64_t r, int64_t j)
@@ -95,12 +97,14 @@ __device__ __forceinline__ uint32_t p_raw_bits(const PDesc &p, const float *base
     if (r >= R || k >= K) return 0u;
     if (p.kind == P_DENSE) return f2u(base[r * p.sr + k * p.sk]);
     int b, y, x, fy, fx, c;
+    // (R and K are below 2^31 on every path that gathers: 32-bit divisions)
+    const uint32_t r32 = (uint32_t)r, k32 = (uint32_t)k, gw = (uint32_t)p.GW, gh = (uint32_t)p.GH, ch = (uint32_t)p.C;
     if (p.kind == P_PATCH) {
-        x = (int)(r % p.GW); const int64_t t = r / p.GW; y = (int)(t % p.GH); b = (int)(t / p.GH);
-        c = (int)(k % p.C); const int u = (int)(k / p.C); fx = u % p.KW; fy = u / p.KW;
+        x = (int)(r32 % gw); const uint32_t t = r32 / gw; y = (int)(t % gh); b = (int)(t / gh);
+        c = (int)(k32 % ch); const int u = (int)(k32 / ch); fx = u % p.KW; fy = u / p.KW;
     } else {
-        c = (int)(r % p.C); const int u = (int)(r / p.C); fx = u % p.KW; fy = u / p.KW;
-        x = (int)(k % p.GW); const int64_t t = k / p.GW; y = (int)(t % p.GH); b = (int)(t / p.GH);
+        c = (int)(r32 % ch); const int u = (int)(r32 / ch); fx = u % p.KW; fy = u / p.KW;
+        x = (int)(k32 % gw); const uint32_t t = k32 / gw; y = (int)(t % gh); b = (int)(t / gh);
     }
     const int iy = y * p.sy - p.pt + fy, ix = x * p.sx - p.pl + fx;
     if ((unsigned)iy >= (unsigned)p.SH || (unsigned)ix >= (unsigned)p.SW) return 0u;

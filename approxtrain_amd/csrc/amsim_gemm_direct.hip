@@ -76,16 +76,17 @@ __device__ __forceinline__ RowRef make_row(const PDesc &p, int64_t r, int64_t R)
     RowRef rr{0, 0, 0, r < R};
     if (!rr.valid) return rr;
     if (PK == P_PATCH) {
-        const int x = (int)(r % p.GW);
-        const int64_t t = r / p.GW;
-        const int y = (int)(t % p.GH);
-        const int b = (int)(t / p.GH);
+        const uint32_t r32 = (uint32_t)r, gw = (uint32_t)p.GW, gh = (uint32_t)p.GH;  // (fewer than 2^31 rows)
+        const int x = (int)(r32 % gw);
+        const uint32_t t = r32 / gw;
+        const int y = (int)(t % gh);
+        const int b = (int)(t / gh);
         rr.vy0 = y * p.sy - p.pt;
         rr.vx0 = x * p.sx - p.pl;
         rr.base = ((b * p.SH + rr.vy0) * p.SW + rr.vx0) * p.C;
     } else if (PK == P_GF) {
-        const int c = (int)(r % p.C);
-        const int t = (int)(r / p.C);
+        const int c = (int)((uint32_t)r % (uint32_t)p.C);
+        const int t = (int)((uint32_t)r / (uint32_t)p.C);
         rr.vx0 = t % p.KW;
         rr.vy0 = t / p.KW;
         rr.base = (rr.vy0 * p.SW + rr.vx0) * p.C + c;
@@ -102,15 +103,15 @@ __device__ __forceinline__ KWalk make_walk(const PDesc &p, int64_t k)
 {
     KWalk w{0, 0, 0};
     if (PK == P_PATCH) {
-        w.c = (int)(k % p.C);
-        const int t = (int)(k / p.C);
+        w.c = (int)((uint32_t)k % (uint32_t)p.C);  // (the reduction is shorter than 2^31)
+        const int t = (int)((uint32_t)k / (uint32_t)p.C);
         w.b = t % p.KW;
         w.a = t / p.KW;
     } else if (PK == P_GF) {
-        w.c = (int)(k % p.GW);
-        const int64_t t = k / p.GW;
-        w.b = (int)(t % p.GH);
-        w.a = (int)(t / p.GH);
+        w.c = (int)((uint32_t)k % (uint32_t)p.GW);
+        const uint32_t t = (uint32_t)k / (uint32_t)p.GW;
+        w.b = (int)(t % (uint32_t)p.GH);
+        w.a = (int)(t / (uint32_t)p.GH);
     }
     return w;
 }
