@@ -276,11 +276,22 @@ __global__ __launch_bounds__(WG_THREADS, 4) void lutgemm_direct_kernel(DArgs a)
 #pragma unroll
                     for (int g = 0; g < G; ++g) {
                         const uint32_t pv = praw[nb * KB + (g0 + g) / TN];
-                        dst[g] = lut_s[__builtin_amdgcn_ubfe(pv, (uint32_t)mshift, (uint32_t)m) + (words[g] & 0x7fffffu)];
+                        // LUT address = lane mantissa index + the word's row offset.  A 16-bit add does it without
+                        // masking the word first: the row offset (< 2^15) sits in its low half, the sign|exponent
+                        // bits drop out, and the instruction clears the upper half of its destination.
+                        uint32_t li;
+                        asm("v_add_u16 %0, %1, %2" : "=v"(li) : "s"(words[g]), "v"(__builtin_amdgcn_ubfe(pv, (uint32_t)mshift, (uint32_t)m)));
+                        dst[g] = lut_s[li];
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 };
-                auto finish_group = [&](int g0, const uint32_t (&src)[G], const uint32_t (&words)[G]) {
+                auto finish_group = [&](int g0, const uint32_t (&src)[G], const uint32_t (&words)[G], bool next_in_flight) {
+                    // one wait for the whole group (all but the next group's G gathers have landed) instead of
+                    // one before every product: each wait is an issue slot of a wavefront that has few to spare
+                    // (operand: no wait on the vector-memory and export counters, LDS counter in bits 11..8)
+                    if (next_in_flight) __builtin_amdgcn_s_waitcnt(0xC07F | (G << 8));
+                    else __builtin_amdgcn_s_waitcnt(0xC07F);
+                    __builtin_amdgcn_sched_barrier(0);  // (keeps the wait ahead of the group's products)
 #pragma unroll
                     for (int g = 0; g < G; ++g) {
                         const uint32_t pv = praw[nb * KB + (g0 + g) / TN];
@@ -294,7 +305,7 @@ __global__ __launch_bounds__(WG_THREADS, 4) void lutgemm_direct_kernel(DArgs a)
 #pragma unroll
                 for (int g0 = 0; g0 < PAIRS; g0 += G) {
                     if (g0 + G < PAIRS) gather_group(g0 + G, lb[((g0 / G) + 1) & 1], sw[((g0 / G) + 1) & 1]);
-                    finish_group(g0, lb[(g0 / G) & 1], sw[(g0 / G) & 1]);
+                    finish_group(g0, lb[(g0 / G) & 1], sw[(g0 / G) & 1], g0 + G < PAIRS);
                 }
             }
         } else {
