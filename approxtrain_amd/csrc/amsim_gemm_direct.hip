@@ -443,11 +443,14 @@ void launch_direct_tn(const DArgs &a, dim3 grid, hipStream_t stream)
 }  // namespace
 
 // Problems the direct engine takes when engines are picked per problem (measured against the
-// LDS-table engine on an MI355X over dense, patch and filter-gradient shapes): up to DIRECT_MAX_MACS
-// padded products, where it wins by 5-45 % (the two meet between 230 and 270 million, beyond 300
-// million the LDS-table engine is ahead); not single- or two-column outputs of a row-major lane
-// operand, whose rows it would read with one strided request per lane.  With any_size (the "direct"
-// engine mode, for tests and tuning) everything it can index.
+// LDS-table engine on an MI355X over dense, patch and filter-gradient shapes, both timed from
+// captured graphs).  The narrower the output, the longer it stays ahead: the LDS-table engine keeps a
+// workgroup's four wavefronts busy only with 32 columns or more.  Up to DIRECT_MAX_MACS_NARROW padded
+// products for at most 8 columns (it wins by 25-45 % there), DIRECT_MAX_MACS_16 for at most 16
+// (10-35 %; the two meet near 230 million), DIRECT_MAX_MACS beyond (the LDS-table engine is ahead
+// from about 60 million on); not single- or two-column outputs of a row-major lane operand, whose
+// rows it would read with one strided request per lane.  With any_size (the "direct" engine mode,
+// for tests and tuning) everything it can index.
 bool direct_shape_eligible(int64_t R, int64_t J, int64_t K, int batch, bool any_size)
 {
     if (K <= 0 || R <= 0 || J <= 0 || batch <= 0) return false;
@@ -455,7 +458,7 @@ bool direct_shape_eligible(int64_t R, int64_t J, int64_t K, int batch, bool any_
     const double tiles = (double)((R + 63) / 64) * (double)((J + tn - 1) / tn) * batch;
     const double padded = tiles * 64.0 * tn * (double)K;
     if (any_size) return padded <= DIRECT_MAX_MACS_ANY;
-    return padded <= DIRECT_MAX_MACS;
+    return padded <= (J <= 8 ? DIRECT_MAX_MACS_NARROW : J <= 16 ? DIRECT_MAX_MACS_16 : DIRECT_MAX_MACS);
 }
 
 bool direct_eligible(int m, const GemmDesc &d, bool any_size)

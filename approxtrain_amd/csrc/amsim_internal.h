@@ -144,7 +144,9 @@ size_t gemm_workspace_bytes_wide(int64_t R, int64_t J, int64_t K, int batch, int
 
 // ---- the direct engine for small problems (one launch, operands read where they lie) ----------
 // Tables that fit the LDS only; which problems it takes is decided in direct_eligible().
-constexpr double DIRECT_MAX_MACS = 200.0e6;
+constexpr double DIRECT_MAX_MACS = 48.0e6;          // padded products; outputs of more than 16 columns
+constexpr double DIRECT_MAX_MACS_16 = 200.0e6;       // ... of 9 to 16 columns
+constexpr double DIRECT_MAX_MACS_NARROW = 400.0e6;   // ... of at most 8 columns
 constexpr double DIRECT_MAX_MACS_ANY = 1.0e10;
 bool direct_shape_eligible(int64_t R, int64_t J, int64_t K, int batch, bool any_size);
 bool direct_eligible(int m, const GemmDesc &d, bool any_size);
