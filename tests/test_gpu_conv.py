@@ -59,6 +59,9 @@ CASES = [
     ((2, 8, 8, 16), (1, 1, 16, 24), 1, "VALID"),      # 1x1
     ((2, 6, 6, 8), (6, 6, 8, 10), 1, "VALID"),        # full-window
     ((1, 11, 13, 5), (4, 3, 5, 7), 3, "SAME"),
+    ((8, 8, 8, 128), (1, 1, 128, 320), 1, "VALID"),   # few pixels, many channels (late ResNet stages): the
+    ((4, 8, 8, 96), (3, 3, 96, 128), 1, "SAME"),      # reduction-slice arrangement under the LDS-table engine
+    ((4, 16, 16, 64), (1, 1, 64, 160), 2, "VALID"),   # ... and a strided 1x1 (three pixel classes in four unreached)
 ]
 
 
