@@ -23,7 +23,7 @@ def lib_path():
 
 _i, _i64, _sz, _p, _f = C.c_int, C.c_int64, C.c_size_t, C.c_void_p, C.c_void_p
 
-# name -> (restype, argtypes); mirrors include/amsim.h declaration by declaration
+# name -> (restype, argtypes); mirrors include/amsim.h and include/amsim_bench.h declaration by declaration
 SIGNATURES = {
     "amsim_status_string": (C.c_char_p, [_i]),
     "amsim_last_error": (C.c_char_p, []),
@@ -39,6 +39,7 @@ SIGNATURES = {
     "amsim_lut_generate_builtin": (_i, [C.c_char_p, _i, _i, _p, _sz]),
     "amsim_mul_f32": (_i, [_p, _f, _f, _f, _sz, _p]),
     "amsim_gemm_workspace_bytes": (_sz, [_i, _i, _i64, _i64, _i64, _i64]),
+    "amsim_gemm_workspace_bytes_for": (_sz, [_p, _i, _i, _i64, _i64, _i64, _i64]),
     "amsim_gemm_plan_info": (_i, [_i, _i, _i64, _i64, _i64, _i64, C.POINTER(_i64)]),
     "amsim_gemm_f32": (_i, [_p, _i, _i, _i, _i64, _i64, _i64, _f, _i64, _f, _i64, _f, _i64,
                             _i64, _i64, _i64, _i64, _p, _sz, _p]),
@@ -55,15 +56,19 @@ SIGNATURES = {
     "amsim_convam_filter_grad_workspace_bytes_for": (_sz, [_p] + [_i] * 7),
     "amsim_convam_filter_grad_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p, _sz, _p]),
     "amsim_denseam_workspace_bytes": (_sz, [_i] * 3),
+    "amsim_denseam_workspace_bytes_for": (_sz, [_p] + [_i] * 3),
     "amsim_denseam_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),
     "amsim_denseam_bias_act_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _f, _i, _p, _sz, _p]),
     "amsim_denseam_weight_grad_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),
     "amsim_denseam_input_grad_f32": (_i, [_p, _f, _f, _f, _i, _i, _i, _p, _sz, _p]),
     "amsim_matmulam_workspace_bytes": (_sz, [_i] * 6),
+    "amsim_matmulam_workspace_bytes_for": (_sz, [_p] + [_i] * 6),
     "amsim_matmulam_f32": (_i, [_p, _f, _f] + [_i] * 6 + [_f, _p, _sz, _p]),
     "amsim_attention_workspace_bytes": (_sz, [_i] * 5),
+    "amsim_attention_workspace_bytes_for": (_sz, [_p] + [_i] * 5),
     "amsim_attention_f32": (_i, [_p, _f, _f, _f, _f, _i, _i64, _i64] + [_i] * 5 + [C.c_float, _f, _f, _p, _sz, _p]),
     "amsim_attention_grad_workspace_bytes": (_sz, [_i] * 5),
+    "amsim_attention_grad_workspace_bytes_for": (_sz, [_p] + [_i] * 5),
     "amsim_attention_grad_f32": (_i, [_p, _f, _f, _f, _f, _f] + [_i] * 5 + [C.c_float, _f, _f, _f, _p, _sz, _p]),
     "amsim_conv_geometry": (_i, [_i, _i, _i, _i, C.POINTER(_i), C.POINTER(_i)]),
     "amsim_set_split_k": (_i, [_i]),

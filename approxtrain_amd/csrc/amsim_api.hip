@@ -2,6 +2,7 @@
 // (which operand runs over the lanes, which is wave-uniform, how the lane
 // operand is gathered) and launches it.  No device memory is allocated here.
 #include "amsim_internal.h"
+#include "amsim_bench.h"
 
 #include <algorithm>
 #include <mutex>
@@ -97,11 +98,15 @@ int gemm_call(amsim_lut_t lut, const GemmCall &g, void *ws, size_t ws_bytes, voi
     return run_gemm(lut->l, describe(g, lut->l.m > 7), ws, ws_bytes, static_cast<hipStream_t>(stream));
 }
 
-size_t gemm_ws(const GemmCall &g)
+// lut == nullptr: valid for any table (the orientation, and with it the engine, depends on the table's
+// width: the larger of both); else what calls through that handle need -- tables that fit the LDS
+// never read the row-staged engine's transposed operand copy, most of the table-agnostic figure.
+size_t gemm_ws(const GemmCall &g, amsim_lut_t lut = nullptr)
 {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0 || g.batch <= 0) return 0;
-    // valid for any table: the orientation (and with it the engine) depends on the table's width
     const GemmDesc d = describe(g, false), w = describe(g, true);
+    if (lut != nullptr && lut->l.m <= 7) return gemm_workspace_bytes(d.R, d.J, d.K, d.batch, d.q.batches);
+    if (lut != nullptr) return gemm_workspace_bytes_any_lut(w.R, w.J, w.K, w.batch, w.q.batches);
     return std::max(gemm_workspace_bytes_any_lut(d.R, d.J, d.K, d.batch, d.q.batches),
                     gemm_workspace_bytes_any_lut(w.R, w.J, w.K, w.batch, w.q.batches));
 }
@@ -138,6 +143,13 @@ size_t amsim_gemm_workspace_bytes(int transA, int transB, int64_t M, int64_t N, 
     // sized for per-item operands (no broadcast), the larger case
     GemmCall g{transA, transB, 0, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, batch, 1, 1, 1};
     return gemm_ws(g);
+}
+
+size_t amsim_gemm_workspace_bytes_for(amsim_lut_t lut, int transA, int transB, int64_t M, int64_t N, int64_t K,
+                                      int64_t batch)
+{
+    GemmCall g{transA, transB, 0, M, N, K, nullptr, 0, nullptr, 0, nullptr, 0, batch, 1, 1, 1};
+    return gemm_ws(g, lut);
 }
 
 int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t info[8])
@@ -458,26 +470,32 @@ GemmCall pointwise_filter_grad(int64_t pixels, int in_depth, int out_depth, cons
 }
 }  // namespace
 
-size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth,
-                                                int filter_rows, int filter_cols, int in_depth)
+namespace {
+size_t filter_grad_ws(amsim_lut_t lut, int batch, int out_rows, int out_cols, int out_depth, int filter_rows,
+                      int filter_cols, int in_depth)
 {
     size_t need = gemm_workspace_bytes((int64_t)filter_rows * filter_cols * in_depth, out_depth,
                                        (int64_t)batch * out_rows * out_cols, 1, 1);
     if (filter_rows == 1 && filter_cols == 1)
         need = std::max(need, gemm_ws(pointwise_filter_grad((int64_t)batch * out_rows * out_cols, in_depth, out_depth,
-                                                            nullptr, nullptr, nullptr)));
+                                                            nullptr, nullptr, nullptr), lut));
+    else if (need && lut != nullptr && lut->l.m > 7)
+        need = std::max(need, gemm_workspace_bytes_wide((int64_t)filter_rows * filter_cols * in_depth, out_depth,
+                                                        (int64_t)batch * out_rows * out_cols, 1, 1));
     return need;
+}
+}  // namespace
+
+size_t amsim_convam_filter_grad_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth,
+                                                int filter_rows, int filter_cols, int in_depth)
+{
+    return filter_grad_ws(nullptr, batch, out_rows, out_cols, out_depth, filter_rows, filter_cols, in_depth);
 }
 
 size_t amsim_convam_filter_grad_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols,
                                                     int out_depth, int filter_rows, int filter_cols, int in_depth)
 {
-    size_t need = amsim_convam_filter_grad_workspace_bytes(batch, out_rows, out_cols, out_depth, filter_rows,
-                                                           filter_cols, in_depth);
-    if (need && lut != nullptr && lut->l.m > 7 && !(filter_rows == 1 && filter_cols == 1))
-        need = std::max(need, gemm_workspace_bytes_wide((int64_t)filter_rows * filter_cols * in_depth, out_depth,
-                                                        (int64_t)batch * out_rows * out_cols, 1, 1));
-    return need;
+    return filter_grad_ws(lut, batch, out_rows, out_cols, out_depth, filter_rows, filter_cols, in_depth);
 }
 
 int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const float *grad, int input_rows,
@@ -518,13 +536,18 @@ int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const floa
 
 // ---- dense ----------------------------------------------------------------------------
 
-size_t amsim_denseam_workspace_bytes(int batch, int units, int input_width)
+size_t amsim_denseam_workspace_bytes_for(amsim_lut_t lut, int batch, int units, int input_width)
 {
     // the largest of the three GEMMs of the layer
     GemmCall f{0, 0, 0, batch, units, input_width, nullptr, 0, nullptr, 0, nullptr, 0, 1, 0, 0, 0};
     GemmCall w{1, 0, 0, input_width, units, batch, nullptr, 0, nullptr, 0, nullptr, 0, 1, 0, 0, 0};
     GemmCall x{0, 1, 1, batch, input_width, units, nullptr, 0, nullptr, 0, nullptr, 0, 1, 0, 0, 0};
-    return std::max(gemm_ws(f), std::max(gemm_ws(w), gemm_ws(x)));
+    return std::max(gemm_ws(f, lut), std::max(gemm_ws(w, lut), gemm_ws(x, lut)));
+}
+
+size_t amsim_denseam_workspace_bytes(int batch, int units, int input_width)
+{
+    return amsim_denseam_workspace_bytes_for(nullptr, batch, units, input_width);
 }
 
 int amsim_denseam_f32(amsim_lut_t lut, const float *inputs, const float *weights, float *output, int batch,
@@ -580,11 +603,17 @@ static int matmul_call(int batch_a, int batch_b, int row_a, int col_a, int row_b
     return AMSIM_OK;
 }
 
-size_t amsim_matmulam_workspace_bytes(int batch_a, int batch_b, int row_a, int col_a, int row_b, int col_b)
+size_t amsim_matmulam_workspace_bytes_for(amsim_lut_t lut, int batch_a, int batch_b, int row_a, int col_a, int row_b,
+                                          int col_b)
 {
     GemmCall g;
     if (matmul_call(batch_a, batch_b, row_a, col_a, row_b, col_b, &g) != AMSIM_OK) return 0;
-    return gemm_ws(g);
+    return gemm_ws(g, lut);
+}
+
+size_t amsim_matmulam_workspace_bytes(int batch_a, int batch_b, int row_a, int col_a, int row_b, int col_b)
+{
+    return amsim_matmulam_workspace_bytes_for(nullptr, batch_a, batch_b, row_a, col_a, row_b, col_b);
 }
 
 int amsim_matmulam_f32(amsim_lut_t lut, const float *a, const float *b, int batch_a, int batch_b, int row_a,
@@ -637,11 +666,16 @@ size_t align256(size_t b) { return (b + 255) / 256 * 256; }
 
 }  // namespace
 
-size_t amsim_attention_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v)
+size_t amsim_attention_workspace_bytes_for(amsim_lut_t lut, int batch, int seq_q, int seq_k, int d_k, int d_v)
 {
     const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
     if (!attn_shape_ok(s)) return 0;
-    return std::max(gemm_ws(s.scores(nullptr, nullptr, nullptr)), gemm_ws(s.context(nullptr, nullptr, nullptr)));
+    return std::max(gemm_ws(s.scores(nullptr, nullptr, nullptr), lut), gemm_ws(s.context(nullptr, nullptr, nullptr), lut));
+}
+
+size_t amsim_attention_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v)
+{
+    return amsim_attention_workspace_bytes_for(nullptr, batch, seq_q, seq_k, d_k, d_v);
 }
 
 int amsim_attention_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *mask,
@@ -665,15 +699,20 @@ int amsim_attention_f32(amsim_lut_t lut, const float *q, const float *k, const f
     return gemm_call(lut, s.context(weights, v, out), workspace, workspace_bytes, stream);
 }
 
-size_t amsim_attention_grad_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v)
+size_t amsim_attention_grad_workspace_bytes_for(amsim_lut_t lut, int batch, int seq_q, int seq_k, int d_k, int d_v)
 {
     const AttnShape s{batch, seq_q, seq_k, d_k, d_v};
     if (!attn_shape_ok(s)) return 0;
-    size_t g = gemm_ws(s.grad_weights(nullptr, nullptr, nullptr));
-    g = std::max(g, gemm_ws(s.grad_v(nullptr, nullptr, nullptr)));
-    g = std::max(g, gemm_ws(s.grad_q(nullptr, nullptr, nullptr)));
-    g = std::max(g, gemm_ws(s.grad_k(nullptr, nullptr, nullptr)));
+    size_t g = gemm_ws(s.grad_weights(nullptr, nullptr, nullptr), lut);
+    g = std::max(g, gemm_ws(s.grad_v(nullptr, nullptr, nullptr), lut));
+    g = std::max(g, gemm_ws(s.grad_q(nullptr, nullptr, nullptr), lut));
+    g = std::max(g, gemm_ws(s.grad_k(nullptr, nullptr, nullptr), lut));
     return align256((size_t)batch * (size_t)s.nw() * sizeof(float)) + g;
+}
+
+size_t amsim_attention_grad_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v)
+{
+    return amsim_attention_grad_workspace_bytes_for(nullptr, batch, seq_q, seq_k, d_k, d_v);
 }
 
 int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *weights,
@@ -686,7 +725,7 @@ int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, co
     if (!attn_shape_ok(s)) return fail(AMSIM_ERR_INVALID, "negative extent");
     if (!(divisor > 0.0f)) return fail(AMSIM_ERR_INVALID, "the score divisor must be positive");
     if (batch == 0) return AMSIM_OK;
-    const size_t need = amsim_attention_grad_workspace_bytes(batch, seq_q, seq_k, d_k, d_v);
+    const size_t need = amsim_attention_grad_workspace_bytes_for(lut, batch, seq_q, seq_k, d_k, d_v);
     if (need && (workspace == nullptr || ((uintptr_t)workspace & 255) || workspace_bytes < need))
         return fail(AMSIM_ERR_WORKSPACE, "workspace missing, not 256-byte aligned or smaller than " +
                                              std::to_string(need) + " bytes");

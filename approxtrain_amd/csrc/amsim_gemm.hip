@@ -914,19 +914,20 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
 // Plans are pure functions of their arguments; the last few are remembered per thread so that
 // the workspace query and the call that follows it do not repeat the search.
 // waves64: waves per SIMD the 64-row kernel variant that will run is compiled for
-static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64)
+// cus: compute units of the machine the plan is for (0 = the current device)
+static Plan make_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int cus = 0)
 {
     struct Key { int64_t R, J, K; int batch, qb, split; };
     struct Slot { Key k; Plan p; bool used = false; };
-    static thread_local Slot memo[8];
+    static thread_local Slot memo[16];
     static thread_local unsigned next = 0;
-    const int cus = device_compute_units();
+    if (cus <= 0) cus = device_compute_units();
     const Key key{R, J, K, batch, q_batches, (split_k ? 1 : 0) | (waves64 << 1) | (cus << 8)};
     for (const Slot &sl : memo)
         if (sl.used && sl.k.R == R && sl.k.J == J && sl.k.K == K && sl.k.batch == batch && sl.k.qb == q_batches &&
             sl.k.split == key.split)
             return sl.p;
-    Slot &sl = memo[next++ % 8];
+    Slot &sl = memo[next++ % 16];
     sl.k = key;
     sl.p = compute_plan(R, J, K, batch, q_batches, split_k, waves64, cus);
     sl.used = true;
@@ -1014,13 +1015,16 @@ static Plan compute_plan(int64_t R, int64_t J, int64_t K, int batch, int q_batch
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 {
     if (R <= 0 || J <= 0 || K <= 0 || batch <= 0) return 0;
-    // valid whichever way amsim_set_split_k stands when the call is made and whichever kernel
-    // variant (6 or 5 waves per SIMD) the operand layout selects
+    // valid whichever way amsim_set_split_k stands when the call is made, whichever kernel variant
+    // (6 or 5 waves per SIMD) the operand layout selects, and -- since the query may be made with no
+    // device or another device current -- for every machine size the plans are made for: the
+    // current device's compute units, 256 (MI355X) and 304
     size_t need = make_plan(R, J, K, batch, q_batches, false, WAVES_PER_SIMD).total;
-    for (int w = WAVES_PER_SIMD - 1; w <= WAVES_PER_SIMD; ++w)
-        need = std::max(need, make_plan(R, J, K, batch, q_batches, true, w).total);
+    for (int cus : {device_compute_units(), 256, 304})
+        for (int w = WAVES_PER_SIMD - 1; w <= WAVES_PER_SIMD; ++w)
+            need = std::max(need, make_plan(R, J, K, batch, q_batches, true, w, cus).total);
     if (direct_shape_eligible(R, J, K, batch, true)) need = std::max(need, direct_workspace_bytes(R, J, K, batch));
-    if (batch == 1 && R <= KLANES_MAX_ROWS && R * J <= KLANES_MAX_OUTPUTS && K >= KLANES_MIN_REDUCTION) need = std::max(need, klanes_workspace_bytes(R, J, K));
+    if (klanes_shape_eligible(R, J, K, batch)) need = std::max(need, klanes_workspace_bytes(R, J, K));
     return need;
 }
 

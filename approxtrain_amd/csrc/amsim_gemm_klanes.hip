@@ -108,7 +108,9 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_klanes_kernel(KLArgs a)
         const int64_t k = k0 + lane;
         const bool valid = wave_live && k < kend;
         const int iy0 = oy * a.p.sy - a.p.pt, ix0 = ox * a.p.sx - a.p.pl;
-        const int pix = ((b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C;
+        // (modulo 2^32: lanes past the slice's end carry an image index beyond the batch, whose offset would
+        // overflow a signed int; it is never dereferenced, and for valid lanes the wrapped sum is the offset)
+        const uint32_t pix = (((uint32_t)b * (uint32_t)a.p.SH + (uint32_t)iy0) * (uint32_t)a.p.SW + (uint32_t)ix0) * (uint32_t)a.p.C;
         const float *qrow = a.q + k * a.q_sk + j0;
         if (JB % 2 == 0 && pairs) {  // whole block inside the row, 8-byte aligned: two channels per load
 #pragma unroll
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(WG_THREADS) void lutgemm_klanes_kernel(KLArgs a)
         for (int rr = 0; rr < RB; ++rr) {
             const bool ok = valid && r0 + rr < a.R && (unsigned)(iy0 + tap_fy[rr]) < (unsigned)a.p.SH &&
                             (unsigned)(ix0 + tap_fx[rr]) < (unsigned)a.p.SW;
-            xr[rr] = ok ? f2u(a.p.base[pix + tap_off[rr]]) : 0u;
+            xr[rr] = ok ? f2u(a.p.base[pix + (uint32_t)tap_off[rr]]) : 0u;
         }
         // on to the pixel of the next pass
         if (stepwise) {
@@ -266,11 +268,15 @@ void launch_klanes_rb(const KLArgs &a, int JB, dim3 grid, hipStream_t stream)
 // (With more filter elements the rows-over-lanes engines win: their gathers stay inside one table row
 // and run conflict-free at about 3.4x the rate of this kernel's scattered ones -- LeNet-5's second
 // convolution, 150 filter elements x 16 channels, takes 31 us there and 39 us here.)
+bool klanes_shape_eligible(int64_t R, int64_t J, int64_t K, int batch)
+{
+    return batch == 1 && R <= KLANES_MAX_ROWS && R * J <= KLANES_MAX_OUTPUTS && K >= KLANES_MIN_REDUCTION && K < (1ll << 31);
+}
+
 bool klanes_eligible(int m, const GemmDesc &d)
 {
-    if (m < 2 || m > 7 || d.p.kind != P_GF || d.q.kind != Q_DENSE || d.q.sj != 1 || d.q.batches != 1 || d.batch != 1)
-        return false;
-    if (d.R > KLANES_MAX_ROWS || d.R * d.J > KLANES_MAX_OUTPUTS || d.K < KLANES_MIN_REDUCTION || d.K >= (1ll << 31)) return false;
+    if (m < 2 || m > 7 || d.p.kind != P_GF || d.q.kind != Q_DENSE || d.q.sj != 1 || d.q.batches != 1) return false;
+    if (!klanes_shape_eligible(d.R, d.J, d.K, d.batch)) return false;
     return (int64_t)d.p.B * d.p.SH * d.p.SW * d.p.C < (1ll << 31);
 }
 

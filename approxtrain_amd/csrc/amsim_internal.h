@@ -159,6 +159,8 @@ int run_gemm_direct(const Lut &lut, const GemmDesc &d, bool may_split, void *wor
 constexpr int64_t KLANES_MAX_ROWS = 32;
 constexpr int64_t KLANES_MAX_OUTPUTS = 4096;
 constexpr int64_t KLANES_MIN_REDUCTION = 2048;
+// the shape part of klanes_eligible (what the workspace query can know)
+bool klanes_shape_eligible(int64_t R, int64_t J, int64_t K, int batch);
 bool klanes_eligible(int m, const GemmDesc &d);
 size_t klanes_workspace_bytes(int64_t R, int64_t J, int64_t K);
 int run_gemm_klanes(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspace_bytes, hipStream_t stream);

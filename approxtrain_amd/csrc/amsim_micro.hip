@@ -5,6 +5,7 @@
 //     second) for the access shapes the kernel could use.
 // They are what the roofline of the bench is priced against.
 #include "amsim_internal.h"
+#include "amsim_bench.h"
 
 #include <algorithm>
 

@@ -74,7 +74,7 @@ def gemm(lut, A, B, trans_a=False, trans_b=False, swap_operands=False):
     batched = A.dim() == 3 or B.dim() == 3
     out = torch.empty((batch, M, N) if batched else (M, N), dtype=torch.float32, device=A.device)
     lib = load_library()
-    nbytes = lib.amsim_gemm_workspace_bytes(int(trans_a), int(trans_b), M, N, K, batch)
+    nbytes = lib.amsim_gemm_workspace_bytes_for(lut.handle, int(trans_a), int(trans_b), M, N, K, batch)
     ws, wsp = _workspace(nbytes, A.device)
     check(lib.amsim_gemm_f32(lut.handle, int(trans_a), int(trans_b), int(swap_operands), M, N, K, _ptr(A), ca,
                              _ptr(B), cb, _ptr(out), N, batch, sA, sB, M * N, wsp, nbytes, _stream()))
@@ -178,7 +178,7 @@ def denseam(lut, inputs, weights, bias=None, activation=None):
     lut = _lut(lut)
     out = torch.empty((batch, units), dtype=torch.float32, device=x.device)
     lib = load_library()
-    nbytes = lib.amsim_denseam_workspace_bytes(batch, units, width)
+    nbytes = lib.amsim_denseam_workspace_bytes_for(lut.handle, batch, units, width)
     ws, wsp = _workspace(nbytes, x.device)
     if b is None and act == 0:
         check(lib.amsim_denseam_f32(lut.handle, _ptr(x), _ptr(w), _ptr(out), batch, units, width, wsp, nbytes,
@@ -198,7 +198,7 @@ def denseam_grad(lut, grad, inputs, weights):
         raise ValueError("grad must be [batch, units]")
     dx, dw = torch.empty_like(x), torch.empty_like(w)
     lib = load_library()
-    nbytes = lib.amsim_denseam_workspace_bytes(batch, units, width)
+    nbytes = lib.amsim_denseam_workspace_bytes_for(lut.handle, batch, units, width)
     ws, wsp = _workspace(nbytes, x.device)
     check(lib.amsim_denseam_weight_grad_f32(lut.handle, _ptr(x), _ptr(dy), _ptr(dw), batch, units, width, wsp,
                                             nbytes, _stream()))
@@ -221,7 +221,7 @@ def matmulam(lut, a, b):
     out = torch.empty((nb, ra, cb) if (a.dim() == 3 or b.dim() == 3) else (ra, cb), dtype=torch.float32,
                       device=a.device)
     lib = load_library()
-    nbytes = lib.amsim_matmulam_workspace_bytes(ba, bb, ra, ca, rb, cb)
+    nbytes = lib.amsim_matmulam_workspace_bytes_for(lut.handle, ba, bb, ra, ca, rb, cb)
     ws, wsp = _workspace(nbytes, a.device)
     check(lib.amsim_matmulam_f32(lut.handle, _ptr(a), _ptr(b), ba, bb, ra, ca, rb, cb, _ptr(out), wsp, nbytes,
                                  _stream()))
@@ -284,7 +284,7 @@ def attention(lut, q, k, v, divisor, mask=None):
     weights = torch.empty(lead + (sq, sk), dtype=torch.float32, device=q.device)
     out = torch.empty(lead + (sq, dv), dtype=torch.float32, device=q.device)
     lib = load_library()
-    nbytes = lib.amsim_attention_workspace_bytes(batch, sq, sk, dk, dv)
+    nbytes = lib.amsim_attention_workspace_bytes_for(lut.handle, batch, sq, sk, dk, dv)
     ws, wsp = _workspace(nbytes, q.device)
     check(lib.amsim_attention_f32(lut.handle, _ptr(q), _ptr(k), _ptr(v), mptr, mdiv, mbs, mrs, batch, sq, sk, dk, dv,
                                   float(divisor), _ptr(weights), _ptr(out), wsp, nbytes, _stream()))
@@ -304,7 +304,7 @@ def attention_grad(lut, q, k, v, weights, grad_out, divisor):
         batch *= d
     gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     lib = load_library()
-    nbytes = lib.amsim_attention_grad_workspace_bytes(batch, sq, sk, dk, dv)
+    nbytes = lib.amsim_attention_grad_workspace_bytes_for(lut.handle, batch, sq, sk, dk, dv)
     ws, wsp = _workspace(nbytes, q.device)
     check(lib.amsim_attention_grad_f32(lut.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(weights), _ptr(grad_out), batch,
                                        sq, sk, dk, dv, float(divisor), _ptr(gq), _ptr(gk), _ptr(gv), wsp, nbytes,

@@ -19,17 +19,19 @@
 //         -L/opt/rocm/lib -lamdhip64 -o convam_gpu.so        (same for denseam_gpu.so, matmulam.so)
 //
 // Scratch memory.  The C ABI never allocates: every entry point takes a
-// workspace (pre-decoded uniform operand, partial sums of split reductions).
-// The dense and matmul functors of the reference carry no temporary at all and
-// the convolution functors carry an im2col buffer sized for another algorithm,
-// so this bridge keeps one growable device buffer per stream and hands it to
-// every call on that stream.  The host lock is held while a call enqueues its
-// kernels, so the kernels of two ops never interleave inside one buffer; the
-// buffer is replaced (after draining the stream) only when a call needs more
-// than any call before it.  OpKernels that want TensorFlow's allocator to own
-// the scratch can size a temp with the *_workspace_bytes queries instead and
-// call the C ABI directly; the im2col / rsfilter temporaries of convam.cc are
-// unused here and can shrink to one element.
+// workspace (pre-decoded uniform operand, partial sums of split reductions)
+// whose size the matching *_workspace_bytes_for query returns.  The dense and
+// matmul functors of the reference carry no temporary at all and the
+// convolution functors an im2col buffer sized for another algorithm, so each
+// functor here takes a temporary from TensorFlow's own allocator through the
+// Eigen device it is handed: GpuDevice::allocate / deallocate forward to the
+// stream interface TensorFlow installs for the running op (EigenGpuStreamDevice
+// in common_runtime/gpu/gpu_device.cc), which allocates from the op's device
+// allocator -- the functor-level form of OpKernelContext::allocate_temp -- and
+// defers the release until the stream has passed the kernels enqueued before
+// it.  No lock, no hipMalloc, no synchronisation; two ops running concurrently
+// hold separate temporaries.  The im2col / rsfilter temporaries of convam.cc
+// are unused here and can shrink to one element.
 //
 // int32 kernels: the reference registers them (convam.cc:620 etc.) but its
 // device product treats the integers as floats.  They are not provided; the
@@ -39,8 +41,6 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdint>
-#include <map>
-#include <mutex>
 
 #include "tensorflow/core/framework/op_kernel.h"
 #include "tensorflow/core/platform/logging.h"
@@ -56,27 +56,28 @@ using tensorflow::int32;
 
 namespace {
 
-// ---- per-stream scratch ------------------------------------------------------
-struct Scratch {
-    void *ptr = nullptr;
-    size_t bytes = 0;
-};
-std::mutex g_lock;                       // held from "get scratch" until the call's kernels are enqueued
-std::map<hipStream_t, Scratch> g_scratch;
+// ---- scratch from TensorFlow's allocator, for the duration of one functor call -------------
+class Scratch {
+public:
+    Scratch(const GPUDevice &d, size_t bytes) : d_(d), bytes_(bytes)
+    {
+        if (bytes_ == 0) return;
+        raw_ = d_.allocate(bytes_ + 256);  // the C ABI wants 256-byte alignment; the allocator promises less
+        if (raw_ == nullptr) LOG(FATAL) << "amsim bridge: cannot allocate " << bytes_ << " bytes of scratch";
+        ptr_ = reinterpret_cast<void *>((reinterpret_cast<uintptr_t>(raw_) + 255) & ~static_cast<uintptr_t>(255));
+    }
+    // handed back once the call's kernels are enqueued: the release is ordered behind them on the stream
+    ~Scratch() { if (raw_) d_.deallocate(raw_); }
+    Scratch(const Scratch &) = delete;
+    Scratch &operator=(const Scratch &) = delete;
+    void *ptr() const { return ptr_; }
+    size_t bytes() const { return bytes_; }
 
-void *scratch_locked(hipStream_t stream, size_t bytes)
-{
-    Scratch &s = g_scratch[stream];
-    if (bytes <= s.bytes) return s.ptr;
-    // kernels already enqueued may still use the old buffer
-    if (hipStreamSynchronize(stream) != hipSuccess) LOG(FATAL) << "amsim bridge: stream synchronize failed";
-    if (s.ptr) (void)hipFree(s.ptr);
-    s = Scratch{};
-    const size_t want = bytes + bytes / 4 + 256;   // head-room: shapes of a model repeat
-    if (hipMalloc(&s.ptr, want) != hipSuccess) LOG(FATAL) << "amsim bridge: cannot allocate " << want << " bytes of scratch";
-    s.bytes = want;
-    return s.ptr;                        // hipMalloc returns 256-byte aligned memory
-}
+private:
+    const GPUDevice &d_;
+    size_t bytes_;
+    void *raw_ = nullptr, *ptr_ = nullptr;
+};
 
 void check(int status, const char *what)
 {
@@ -131,10 +132,10 @@ void ConvamFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const T *input_
     // (the table-aware queries: tables wider than 7 bits also get the staged operand their engine reads)
     const size_t ws = amsim_convam_workspace_bytes_for(handle_of(mul_lut), batch, out_rows, out_cols, out_depth, filter_rows,
                                                        filter_cols, in_depth);
-    std::lock_guard<std::mutex> hold(g_lock);
+    Scratch scratch(d, ws);
     check(amsim_convam_f32(handle_of(mul_lut), input_data, output_data, batch, out_rows, out_cols, out_depth,
                            stride_cols, stride_rows, filter_left_offset, filter_top_offset, filter_rows, filter_cols,
-                           in_depth, input_cols, input_rows, filter, scratch_locked(d.stream(), ws), ws, d.stream()),
+                           in_depth, input_cols, input_rows, filter, scratch.ptr(), scratch.bytes(), d.stream()),
           "Convam");
 }
 template <>
@@ -161,11 +162,11 @@ void ConvamInputGradFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const 
     const size_t ws = amsim_convam_input_grad_workspace_bytes_for(handle_of(mul_lut), batch, input_rows, input_cols,
                                                                   in_depth, filter_rows, filter_cols, out_depth,
                                                                   stride_rows, stride_cols, pad_top, pad_left);
-    std::lock_guard<std::mutex> hold(g_lock);
+    Scratch scratch(d, ws);
     check(amsim_convam_input_grad_f32(handle_of(mul_lut), grad, hole_grad_width, hole_grad_height, pad_top, pad_left,
                                       filter, filter_rows, filter_cols, out_depth, stride_rows, stride_cols, batch,
                                       input_rows, input_cols, in_depth, output, out_rows, out_cols,
-                                      scratch_locked(d.stream(), ws), ws, d.stream()),
+                                      scratch.ptr(), scratch.bytes(), d.stream()),
           "ConvamInputGrad");
 }
 template <>
@@ -190,11 +191,11 @@ void ConvamFilterGradFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const
 {
     const size_t ws = amsim_convam_filter_grad_workspace_bytes_for(handle_of(mul_lut), batch, out_rows, out_cols, out_depth,
                                                                    filter_rows, filter_cols, in_depth);
-    std::lock_guard<std::mutex> hold(g_lock);
+    Scratch scratch(d, ws);
     check(amsim_convam_filter_grad_f32(handle_of(mul_lut), input, grad, input_rows, input_cols, batch, in_depth,
                                        out_cols, out_rows, out_depth, filter_left_offset, filter_top_offset,
                                        stride_rows, stride_cols, filter_cols, filter_rows, output,
-                                       scratch_locked(d.stream(), ws), ws, d.stream()),
+                                       scratch.ptr(), scratch.bytes(), d.stream()),
           "ConvamFilterGrad");
 }
 template <>
@@ -220,10 +221,10 @@ void DenseamFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const T *input
                                               const int batch, const int units, const int input_width,
                                               approx_mul_lut<GPUDevice> &mul_lut)
 {
-    const size_t ws = amsim_denseam_workspace_bytes(batch, units, input_width);
-    std::lock_guard<std::mutex> hold(g_lock);
+    const size_t ws = amsim_denseam_workspace_bytes_for(handle_of(mul_lut), batch, units, input_width);
+    Scratch scratch(d, ws);
     check(amsim_denseam_f32(handle_of(mul_lut), inputs, weights, output, batch, units, input_width,
-                            scratch_locked(d.stream(), ws), ws, d.stream()),
+                            scratch.ptr(), scratch.bytes(), d.stream()),
           "Denseam");
 }
 template <>
@@ -238,10 +239,10 @@ void DenseamWeightGradFunctor<GPUDevice, T>::operator()(const GPUDevice &d, cons
                                                         const int batch, const int units, const int input_width,
                                                         approx_mul_lut<GPUDevice> &mul_lut)
 {
-    const size_t ws = amsim_denseam_workspace_bytes(batch, units, input_width);
-    std::lock_guard<std::mutex> hold(g_lock);
+    const size_t ws = amsim_denseam_workspace_bytes_for(handle_of(mul_lut), batch, units, input_width);
+    Scratch scratch(d, ws);
     check(amsim_denseam_weight_grad_f32(handle_of(mul_lut), input, grads, output, batch, units, input_width,
-                                        scratch_locked(d.stream(), ws), ws, d.stream()),
+                                        scratch.ptr(), scratch.bytes(), d.stream()),
           "DenseamGrad (weights)");
 }
 template <>
@@ -257,10 +258,10 @@ void DenseamInputGradFunctor<GPUDevice, T>::operator()(const GPUDevice &d, const
                                                        const int batch, const int units, const int input_width,
                                                        approx_mul_lut<GPUDevice> &mul_lut)
 {
-    const size_t ws = amsim_denseam_workspace_bytes(batch, units, input_width);
-    std::lock_guard<std::mutex> hold(g_lock);
+    const size_t ws = amsim_denseam_workspace_bytes_for(handle_of(mul_lut), batch, units, input_width);
+    Scratch scratch(d, ws);
     check(amsim_denseam_input_grad_f32(handle_of(mul_lut), weight, grads, output, batch, units, input_width,
-                                       scratch_locked(d.stream(), ws), ws, d.stream()),
+                                       scratch.ptr(), scratch.bytes(), d.stream()),
           "DenseamGrad (inputs)");
 }
 template <>
@@ -287,10 +288,10 @@ void LaunchMatMul<GPUDevice, T>::operator()(const GPUDevice &d, const T *a, cons
                                             const int batch_b, const int row_a, const int col_a, const int row_b,
                                             const int col_b, T *out, approx_mul_lut<GPUDevice> &mul_lut)
 {
-    const size_t ws = amsim_matmulam_workspace_bytes(batch_a, batch_b, row_a, col_a, row_b, col_b);
-    std::lock_guard<std::mutex> hold(g_lock);
+    const size_t ws = amsim_matmulam_workspace_bytes_for(handle_of(mul_lut), batch_a, batch_b, row_a, col_a, row_b, col_b);
+    Scratch scratch(d, ws);
     check(amsim_matmulam_f32(handle_of(mul_lut), a, b, batch_a, batch_b, row_a, col_a, row_b, col_b, out,
-                             scratch_locked(d.stream(), ws), ws, d.stream()),
+                             scratch.ptr(), scratch.bytes(), d.stream()),
           "MatMulAM");
 }
 template <>

@@ -83,7 +83,8 @@ def device_ms(fn, min_reps=3, min_ms=20.0, max_reps=200):
 def device_ms_graph(fn, calls=40, replays=5):
     """Device time of fn() in ms for calls shorter than the host takes to enqueue one (about 18 us from
     Python): `calls` of them are captured into one HIP graph on a side stream and the graph's replay is
-    timed with HIP events (best of `replays`), so the figure holds no host time between launches."""
+    timed with HIP events (median of `replays`, the statistic of the headline step time), so the figure
+    holds no host time between launches."""
     import torch
     s = torch.cuda.Stream()
     with torch.cuda.stream(s):
@@ -97,15 +98,15 @@ def device_ms_graph(fn, calls=40, replays=5):
     torch.cuda.synchronize()
     g.replay()
     torch.cuda.synchronize()
-    best = float("inf")
+    times = []
     for _ in range(replays):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         g.replay()
         e1.record()
         torch.cuda.synchronize()
-        best = min(best, e0.elapsed_time(e1) / calls)
-    return best
+        times.append(e0.elapsed_time(e1) / calls)
+    return statistics.median(times)
 
 
 def _microbench(lib, kind, blocks, sink, wide_table=None):
@@ -323,6 +324,25 @@ def run_cfg5(roof):
     return out
 
 
+RESNET50_SIZES = (("feature_maps_56_to_7", 56, 64), ("feature_maps_32_to_4_cifar", 32, 3))
+
+
+def resnet50_layers(hw0, cin0):
+    """The distinct convolutions of ResNet-50's bottleneck stages 2-5 for an hw0 x hw0 x cin0 input to
+    stage 2: (name, H = W, Cin, Cout, filter size, stride, how many the model holds)."""
+    layers = []
+    hw, cin = hw0, cin0
+    for stage, (f1, f3, nblocks, stride) in enumerate(((64, 256, 3, 1), (128, 512, 4, 2), (256, 1024, 6, 2), (512, 2048, 3, 2)), start=2):
+        ohw = (hw - 1) // stride + 1
+        layers += [("s%da_1x1/%d_%d_%d" % (stage, stride, cin, f1), hw, cin, f1, 1, stride, 1),
+                   ("s%da_shortcut_1x1/%d_%d_%d" % (stage, stride, cin, f3), hw, cin, f3, 1, stride, 1),
+                   ("s%d_3x3_%d_%d" % (stage, f1, f1), ohw, f1, f1, 3, 1, nblocks),
+                   ("s%d_1x1_%d_%d" % (stage, f1, f3), ohw, f1, f3, 1, 1, nblocks),
+                   ("s%d_1x1_%d_%d" % (stage, f3, f1), ohw, f3, f1, 1, 1, nblocks - 1)]
+        hw, cin = ohw, f3
+    return layers
+
+
 def run_resnet50(roof):
     """Every convolution of ResNet-50's bottleneck stages 2-5 (the layout profile/resnet50.py:295-313
     builds: per stage one block with a strided 1x1 and a 1x1 shortcut, then identity blocks of
@@ -336,17 +356,8 @@ def run_resnet50(roof):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(20)
     out = {}
-    for label, hw0, cin0 in (("feature_maps_56_to_7", 56, 64), ("feature_maps_32_to_4_cifar", 32, 3)):
-        layers = []  # (name, H = W, Cin, Cout, k, stride, how many)
-        hw, cin = hw0, cin0
-        for stage, (f1, f3, nblocks, stride) in enumerate(((64, 256, 3, 1), (128, 512, 4, 2), (256, 1024, 6, 2), (512, 2048, 3, 2)), start=2):
-            ohw = (hw - 1) // stride + 1
-            layers += [("s%da_1x1/%d_%d_%d" % (stage, stride, cin, f1), hw, cin, f1, 1, stride, 1),
-                       ("s%da_shortcut_1x1/%d_%d_%d" % (stage, stride, cin, f3), hw, cin, f3, 1, stride, 1),
-                       ("s%d_3x3_%d_%d" % (stage, f1, f1), ohw, f1, f1, 3, 1, nblocks),
-                       ("s%d_1x1_%d_%d" % (stage, f1, f3), ohw, f1, f3, 1, 1, nblocks),
-                       ("s%d_1x1_%d_%d" % (stage, f3, f1), ohw, f3, f1, 1, 1, nblocks - 1)]
-            hw, cin = ohw, f3
+    for label, hw0, cin0 in RESNET50_SIZES:
+        layers = resnet50_layers(hw0, cin0)
         total_ms = total_macs = 0.0
         per_layer = {}
         for name, hw, cin, cout, k, stride, count in layers:

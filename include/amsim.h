@@ -114,6 +114,14 @@ int amsim_mul_f32(amsim_lut_t lut, const float *a, const float *b, float *out, s
  * batch (stride 0 broadcasts an operand), replacing the per-item launch loop
  * of cuda/matmulam_kernel.cu:30-98. */
 size_t amsim_gemm_workspace_bytes(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch);
+/* The query above is an upper bound over every table: it includes the transposed operand copy
+ * that only tables of 8..11 mantissa bits read (the row-staged engine), several times what a
+ * table that fits the LDS needs.  The query for a given table returns what calls through that
+ * handle use; amsim_denseam_ / amsim_matmulam_ / amsim_attention_ / amsim_attention_grad_
+ * workspace_bytes_for below are the same for their entry points.  A NULL handle gives the upper
+ * bound. */
+size_t amsim_gemm_workspace_bytes_for(amsim_lut_t lut, int transA, int transB, int64_t M, int64_t N, int64_t K,
+                                      int64_t batch);
 int amsim_gemm_f32(amsim_lut_t lut, int transA, int transB, int swap_operands, int64_t M, int64_t N,
                    int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                    int64_t ldc, int64_t batch, int64_t strideA, int64_t strideB, int64_t strideC,
@@ -206,6 +214,7 @@ int amsim_convam_filter_grad_f32(amsim_lut_t lut, const float *input, const floa
 
 /* ---- dense functors (denseam.h:9-27, cuda/denseam_kernel.cu:98-145) ---------- */
 size_t amsim_denseam_workspace_bytes(int batch, int units, int input_width);
+size_t amsim_denseam_workspace_bytes_for(amsim_lut_t lut, int batch, int units, int input_width);
 /* DenseamFunctor: output[batch][units] = inputs[batch][input_width] . weights[input_width][units] */
 int amsim_denseam_f32(amsim_lut_t lut, const float *inputs, const float *weights, float *output, int batch,
                       int units, int input_width, void *workspace, size_t workspace_bytes, void *stream);
@@ -227,6 +236,8 @@ int amsim_denseam_input_grad_f32(amsim_lut_t lut, const float *weight, const flo
  * batch_a / batch_b: 0 for a rank-2 operand, else its leading dimension; a
  * batch of 1 broadcasts (matmulam.cc:86-147). */
 size_t amsim_matmulam_workspace_bytes(int batch_a, int batch_b, int row_a, int col_a, int row_b, int col_b);
+size_t amsim_matmulam_workspace_bytes_for(amsim_lut_t lut, int batch_a, int batch_b, int row_a, int col_a, int row_b,
+                                          int col_b);
 int amsim_matmulam_f32(amsim_lut_t lut, const float *a, const float *b, int batch_a, int batch_b, int row_a,
                        int col_a, int row_b, int col_b, float *out, void *workspace, size_t workspace_bytes,
                        void *stream);
@@ -246,6 +257,7 @@ int amsim_matmulam_f32(amsim_lut_t lut, const float *a, const float *b, int batc
  * r * mask_row_stride + j], which covers a mask shared by the heads of one
  * sample (mask_batch_div = heads) and masks broadcast over queries (row stride 0). */
 size_t amsim_attention_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v);
+size_t amsim_attention_workspace_bytes_for(amsim_lut_t lut, int batch, int seq_q, int seq_k, int d_k, int d_v);
 int amsim_attention_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *mask,
                         int mask_batch_div, int64_t mask_batch_stride, int64_t mask_row_stride, int batch, int seq_q,
                         int seq_k, int d_k, int d_v, float divisor, float *weights, float *out, void *workspace,
@@ -256,6 +268,7 @@ int amsim_attention_f32(amsim_lut_t lut, const float *q, const float *k, const f
  * d(scores) = softmax gradient / divisor,  d(q) = d(scores) . k,  d(k) = (q^T . d(scores))^T.
  * The workspace also holds d(scores) (batch * seq_q * seq_k floats). */
 size_t amsim_attention_grad_workspace_bytes(int batch, int seq_q, int seq_k, int d_k, int d_v);
+size_t amsim_attention_grad_workspace_bytes_for(amsim_lut_t lut, int batch, int seq_q, int seq_k, int d_k, int d_v);
 int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, const float *v, const float *weights,
                              const float *grad_out, int batch, int seq_q, int seq_k, int d_k, int d_v, float divisor,
                              float *grad_q, float *grad_k, float *grad_v, void *workspace, size_t workspace_bytes,
@@ -266,7 +279,7 @@ int amsim_attention_grad_f32(amsim_lut_t lut, const float *q, const float *k, co
  * convam.cc:382-387, 553-572, 1071-1084: output extent and leading pad. */
 int amsim_conv_geometry(int in_size, int filter_size, int stride, int padding, int *out_size, int *pad_before);
 
-/* ---- knobs and measurement helpers (no counterpart in the reference) ----------
+/* ---- knobs (no counterpart in the reference) -------------------------------------
  * amsim_set_split_k sets the process default that handles in mode -1 follow (see
  * amsim_lut_set_split_k for the two modes and their tolerance); the initial default is 1. */
 int amsim_set_split_k(int mode);
@@ -283,41 +296,6 @@ int amsim_set_engine(int mode);
 /* The same choice for calls through one handle (-1, the initial value, follows the process-wide
  * setting): lets threads hold different settings without sharing mutable state. */
 int amsim_lut_set_engine(amsim_lut_t lut, int mode);
-/* How a GEMM of this shape would be run when reductions may be split (contiguous, aligned
- * operands assumed): info = {outputs per lane, row tiles per workgroup, splits of the main part's
- * reduction, chunks (of 32) per split, rows in the main part, splits of the tail rows' reduction
- * (0 = no tail), chunks per tail split, chunks in all}.  For tests and tuning. */
-int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t info[8]);
-/* Micro-kernels that measure, on the current device, the VALU issue rate
- * (kind 0 / 10: independent FP32 FMAs; 11..13: v_add_u32, v_lshl_add_u32,
- * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's mix, 5 instructions per two MACs;
- * 16: the row-staged GEMM's pair per product, a 16-bit multiply-add that forms the factor + an FMA) and
- * the LDS gather rate (kinds 1..6: u8 / u16 / b32 reads, lanes inside one
- * 128-element row or scattered, with 64 KB of LDS per workgroup; kinds 21 / 22: the u8 pair
- * again at the GEMM kernel's own LDS footprint and occupancy, reads software-pipelined).
- * Kinds 10..16 also leave two 64-bit counts at sink[512..515]: the shader-clock ticks of one
- * workgroup's loop and the same interval in 100 MHz ticks (their ratio is the clock).  Launches
- * `reps` times on `stream`, timed with HIP events; `sink` is any device buffer
- * of >= 256 floats. */
-int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream, float *sink,
-                     double *ms_per_launch, double *ops_per_launch);
-/* The rates that bound products through tables too wide for the LDS (mantissa widths 8..11,
- * rows of 4 KB in device memory): kind 0 = one 2-byte global gather per product, all lanes of a
- * wavefront inside one random row; 1 = whole random rows pulled into LDS by direct
- * global-to-LDS loads (bytes); 2 = 16-bit LDS gathers with the lanes scattered over 4 KB rows;
- * 3 = 1 and 2 overlapped (64 KB of rows per 65536 products: the shape of a row-staged GEMM that
- * keeps the rows apart in LDS); 4 = 16-byte LDS reads with the lanes scattered over a 32 KB
- * half of interleaved rows, 8 products per read (the row-staged GEMM's gathers); 5 = whole random
- * rows pulled into registers by coalesced 4-byte loads (bytes; the GEMM's own fetches).  `table`
- * is a device buffer of table_bytes >= 8 KB, 16-byte aligned; workgroups have 1024 threads;
- * ops_per_launch counts products (bytes for kinds 1 and 5). */
-int amsim_microbench_wide(int kind, int blocks, int iters, int reps, void *stream, const void *table,
-                          size_t table_bytes, float *sink, double *ms_per_launch, double *ops_per_launch);
-
-/* Plain copy kernel of known size (reads 4n bytes, writes 4n bytes; n % 4 == 0,
- * 16-byte aligned buffers): the reference point that hardware traffic counters
- * (FETCH_SIZE / WRITE_SIZE) are scaled against. */
-int amsim_calibration_copy(const float *src, float *dst, size_t n, void *stream);
 
 #ifdef __cplusplus
 }

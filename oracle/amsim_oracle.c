@@ -24,6 +24,10 @@
  *       every product is exact, so results must equal an integer GEMM / a
  *       library convolution and its autograd bit for bit; and by brute-force
  *       loop nests on tiny shapes.
+ *   amo_gemm_abs (the tolerance normaliser sum|P|)
+ *       pinned: equals |A| . |B| exactly for integer operands under ACC_7 in
+ *       every transpose / operand-order form, and the sum of |amo_lut_mul|
+ *       element by element for the real multiplier and an asymmetric table.
  *   amo_lutgen32 with m > 7 (no reference file or model exists for m = 11):
  *       PARITY UNPINNED beyond the closed-form rules that reproduce m <= 7.
  */
@@ -442,8 +446,9 @@ AMO_EXPORT int amo_matmul(const uint32_t *lut32, int m, const float *a, const fl
 /* sum over the same products of |P(a,b)|, for the 1e-5 * sum|p| tolerance */
 AMO_EXPORT void amo_gemm_abs(const uint32_t *lut32, int m, int transA, int transB, int swap,
                              long M, long N, long K, const float *A, long lda, const float *B,
-                             long ldb, double *C, long ldc)
+                             long ldb, double *C, long ldc, int threads)
 {
+#pragma omp parallel for schedule(static) num_threads(threads > 0 ? threads : 1)
     for (long i = 0; i < M; ++i)
         for (long j = 0; j < N; ++j) {
             double acc = 0.0;

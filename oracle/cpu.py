@@ -98,7 +98,7 @@ def gemm(lut32, m, A, B, transA=False, transB=False, swap=False, threads=1):
     return out
 
 
-def gemm_abs(lut32, m, A, B, transA=False, transB=False, swap=False):
+def gemm_abs(lut32, m, A, B, transA=False, transB=False, swap=False, threads=1):
     """sum_k |P(a,b)| per output, in float64: the tolerance normaliser."""
     A, pa = _f(A)
     B, pb = _f(B)
@@ -108,7 +108,7 @@ def gemm_abs(lut32, m, A, B, transA=False, transB=False, swap=False):
     out = np.zeros((M, N), dtype=np.float64)
     _lib.amo_gemm_abs(_lut(lut32), C.c_int(m), C.c_int(transA), C.c_int(transB), C.c_int(swap),
                       C.c_long(M), C.c_long(N), C.c_long(K), pa, C.c_long(A.shape[1]), pb,
-                      C.c_long(B.shape[1]), out.ctypes.data_as(C.POINTER(C.c_double)), C.c_long(N))
+                      C.c_long(B.shape[1]), out.ctypes.data_as(C.POINTER(C.c_double)), C.c_long(N), C.c_int(threads))
     return out
 
 

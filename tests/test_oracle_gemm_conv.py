@@ -66,6 +66,45 @@ def test_gemm_operand_order_and_accumulation_order():
     assert not np.array_equal(got, got_sw)  # the table really is asymmetric
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("swap", [False, True])
+def test_gemm_abs_is_the_product_of_absolute_integer_matrices(ta, tb, swap):
+    """The tolerance normaliser sum_k |P(a, b)|: with ACC_7 on small integers every product is
+    exact, so the sum must equal |op(A)| . |op(B)| exactly for every transpose form and either
+    operand order (a wrong index or transposition changes it; cancelling signs would too)."""
+    rng = np.random.default_rng(21)
+    M, N, K = 23, 31, 47
+    A = small_ints(rng, (K, M) if ta else (M, K))
+    B = small_ints(rng, (N, K) if tb else (K, N))
+    want = np.abs(A.T if ta else A).astype(np.int64) @ np.abs(B.T if tb else B).astype(np.int64)
+    got = cpu.gemm_abs(ACC7, 7, A, B, transA=ta, transB=tb, swap=swap)
+    assert got.dtype == np.float64 and np.array_equal(got, want.astype(np.float64))
+    # sum|p| >= |sum p|, with equality only where no signs cancel: the signed GEMM differs
+    signed = cpu.gemm(ACC7, 7, A, B, transA=ta, transB=tb, swap=swap).astype(np.float64)
+    assert np.all(got >= np.abs(signed)) and np.any(got > np.abs(signed))
+
+
+def test_gemm_abs_sums_the_lut_products_and_skips_non_finite_ones():
+    """With the real multiplier (MBM_7) and an asymmetric table: the sum of |lut_mul| of every
+    operand pair, in float64; infinite and NaN products are left out (they are compared as a class)."""
+    rng = np.random.default_rng(22)
+    A = rng.standard_normal((6, 13)).astype(np.float32)
+    B = rng.standard_normal((13, 5)).astype(np.float32)
+    A[2, 3], B[4, 1] = np.inf, np.nan
+    for lut, m in ((MBM7, 7), (asym_lut(3), 3)):
+        for swap in (False, True):
+            want = np.zeros((6, 5))
+            for i in range(6):
+                for j in range(5):
+                    a, b = A[i], np.ascontiguousarray(B[:, j])
+                    p = cpu.lut_mul_array(lut, m, b, a) if swap else cpu.lut_mul_array(lut, m, a, b)
+                    p = p.astype(np.float64)
+                    want[i, j] = np.abs(p[np.isfinite(p)]).sum()
+            got = cpu.gemm_abs(lut, m, A, B, swap=swap)
+            assert np.allclose(got, want, rtol=1e-14, atol=0)
+    assert not np.array_equal(cpu.gemm_abs(asym_lut(3), 3, A, B), cpu.gemm_abs(asym_lut(3), 3, A, B, swap=True))
+
+
 def test_dense_fwd_and_grads_exact():
     rng = np.random.default_rng(4)
     x, w, dy = small_ints(rng, (6, 13)), small_ints(rng, (13, 7)), small_ints(rng, (6, 7))
