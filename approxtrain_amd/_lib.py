@@ -45,6 +45,7 @@ SIGNATURES = {
                             _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "amsim_convam_workspace_bytes": (_sz, [_i] * 7),
     "amsim_convam_workspace_bytes_for": (_sz, [_p] + [_i] * 7),
+    "amsim_convam_lean_workspace_bytes_for": (_sz, [_p] + [_i] * 9),
     "amsim_convam_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p, _sz, _p]),
     "amsim_convam_noalloc_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _p]),
     "amsim_convam_bias_act_f32": (_i, [_p, _f, _f] + [_i] * 13 + [_f, _f, _i, _p, _sz, _p]),

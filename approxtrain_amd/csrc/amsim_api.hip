@@ -173,6 +173,30 @@ int amsim_gemm_f32(amsim_lut_t lut, int transA, int transB, int swap_operands, i
 
 // ---- convolution ------------------------------------------------------------------
 
+}  // extern "C"
+
+namespace {
+// im2col rows (b, oy, ox) x columns (fy, fx, c)  [cuda_kernel.cu:35-60], filter as the [K][OC] matrix
+GemmDesc forward_desc(int batch, int out_rows, int out_cols, int out_depth, int stride_cols, int stride_rows,
+                      int filter_left_offset, int filter_top_offset, int filter_rows, int filter_cols, int in_depth,
+                      int input_cols, int input_rows)
+{
+    GemmDesc d;
+    d.R = (int64_t)batch * out_rows * out_cols; d.J = out_depth; d.K = (int64_t)filter_rows * filter_cols * in_depth;
+    d.p.kind = P_PATCH;
+    d.p.B = batch; d.p.GH = out_rows; d.p.GW = out_cols;
+    d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = in_depth;
+    d.p.sy = stride_rows; d.p.sx = stride_cols; d.p.pt = filter_top_offset; d.p.pl = filter_left_offset;
+    d.p.SH = input_rows; d.p.SW = input_cols;
+    d.q.kind = Q_DENSE; d.q.sk = out_depth; d.q.sj = 1;
+    d.so_r = out_depth; d.so_j = 1;
+    d.lane_first = true;  // P(input, filter)
+    return d;
+}
+}  // namespace
+
+extern "C" {
+
 size_t amsim_convam_workspace_bytes(int batch, int out_rows, int out_cols, int out_depth, int filter_rows,
                                     int filter_cols, int in_depth)
 {
@@ -188,6 +212,20 @@ size_t amsim_convam_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows
         need = std::max(need, gemm_workspace_bytes_wide((int64_t)batch * out_rows * out_cols, out_depth,
                                                         (int64_t)filter_rows * filter_cols * in_depth, 1, 1));
     return need;
+}
+
+size_t amsim_convam_lean_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols, int out_depth,
+                                             int filter_rows, int filter_cols, int in_depth, int stride_rows,
+                                             int stride_cols)
+{
+    size_t need = amsim_convam_workspace_bytes(batch, out_rows, out_cols, out_depth, filter_rows, filter_cols, in_depth);
+    if (!need || lut == nullptr || lut->l.m <= 7 || stride_rows < 1 || stride_cols < 1) return need;
+    // (the copy's extent follows from the output extent, the strides and the filter: the source's own
+    // extent and the pads do not enter)
+    const GemmDesc d = forward_desc(batch, out_rows, out_cols, out_depth, stride_cols, stride_rows, 0, 0, filter_rows,
+                                    filter_cols, in_depth, (out_cols - 1) * stride_cols + filter_cols,
+                                    (out_rows - 1) * stride_rows + filter_rows);
+    return std::max(need, gemm_workspace_bytes_wide_planar(d));
 }
 
 int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_data, int batch, int out_rows,
@@ -217,18 +255,12 @@ int amsim_convam_bias_act_f32(amsim_lut_t lut, const float *input_data, float *o
     if (!input_data || !output_data || !filter) return fail(AMSIM_ERR_INVALID, "null tensor pointer");
     if (!fits_int32((int64_t)batch * input_rows * input_cols * in_depth))
         return fail(AMSIM_ERR_UNSUPPORTED, "input tensor has 2^31 or more elements");
-    // im2col rows (b, oy, ox) x columns (fy, fx, c)  [cuda_kernel.cu:35-60], filter as the [K][OC] matrix
-    GemmDesc d;
-    d.R = R; d.J = out_depth; d.K = (int64_t)filter_rows * filter_cols * in_depth;
-    d.p.kind = P_PATCH; d.p.base = input_data;
-    d.p.B = batch; d.p.GH = out_rows; d.p.GW = out_cols;
-    d.p.KH = filter_rows; d.p.KW = filter_cols; d.p.C = in_depth;
-    d.p.sy = stride_rows; d.p.sx = stride_cols; d.p.pt = filter_top_offset; d.p.pl = filter_left_offset;
-    d.p.SH = input_rows; d.p.SW = input_cols;
-    d.q.kind = Q_DENSE; d.q.base = filter; d.q.sk = out_depth; d.q.sj = 1;
-    d.out = output_data; d.so_r = out_depth; d.so_j = 1;
+    GemmDesc d = forward_desc(batch, out_rows, out_cols, out_depth, stride_cols, stride_rows, filter_left_offset,
+                              filter_top_offset, filter_rows, filter_cols, in_depth, input_cols, input_rows);
+    d.p.base = input_data;
+    d.q.base = filter;
+    d.out = output_data;
     d.bias_j = bias; d.act = activation;
-    d.lane_first = true;  // P(input, filter)
     return run_gemm(lut->l, d, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 

@@ -37,6 +37,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cstdlib>
 
 namespace amsim {
 
@@ -747,6 +748,30 @@ __global__ __launch_bounds__(WG_THREADS) void splitk_reduce_kernel(RArgs a)
     }
 }
 
+// Few slices over many outputs whose rows are contiguous (slices of a tall problem's reduction): a
+// thread adds four consecutive columns of one row across the slices, in slice order, with 16-byte
+// loads and one 16-byte store -- the general kernel above spends a workgroup on 64 outputs.
+__global__ __launch_bounds__(WG_THREADS) void splitk_reduce_rows4_kernel(RArgs a)
+{
+    const int64_t idx = (int64_t)blockIdx.x * WG_THREADS + threadIdx.x;
+    const int64_t per_row = a.J / 4;
+    if (idx >= a.R * per_row) return;
+    const int bz = blockIdx.y;
+    const int64_t r = idx / per_row, j = (idx - r * per_row) * 4;
+    const size_t stride = (size_t)a.batch * a.Rp * a.Jp;
+    const float *src = a.partial + ((size_t)bz * a.Rp + r) * a.Jp + j;
+    float4 s = *reinterpret_cast<const float4 *>(src);
+    for (int sp = 1; sp < a.nsplit; ++sp) {
+        const float4 v = *reinterpret_cast<const float4 *>(src + (size_t)sp * stride);
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    s.x = apply_epilogue(a.ep, s.x, a.row_base + r, j);
+    s.y = apply_epilogue(a.ep, s.y, a.row_base + r, j + 1);
+    s.z = apply_epilogue(a.ep, s.z, a.row_base + r, j + 2);
+    s.w = apply_epilogue(a.ep, s.w, a.row_base + r, j + 3);
+    *reinterpret_cast<float4 *>(a.out + (int64_t)bz * a.out_batch_stride + out_row_offset(a.ep.omap, a.row_base + r, a.so_r) + j) = s;
+}
+
 // Empty reduction: every output is the epilogue of zero (zeros without one).  VEC = 4: a thread
 // writes four consecutive columns of a row as one 16-byte store (rows contiguous, 16-byte aligned,
 // a multiple of four columns): the pixel classes of a strided grad-input that no filter tap
@@ -818,6 +843,15 @@ int launch_skipped_tap_poison(const float *filter, int KH, int KW, int IC, int O
 void launch_reduce(const RArgs &ra, hipStream_t stream)
 {
     const int64_t outs = ra.R * ra.J;
+    // (the slices of the general kernel are summed as eight interleaved chains per way; with at most
+    // eight slices and one way per output that is the plain sum in slice order, which this kernel forms too)
+    const bool rows4 = ra.nsplit <= 4 && outs >= (1 << 20) && ra.J % 4 == 0 && ra.Jp % 4 == 0 && ra.so_j == 1 && ra.so_r % 4 == 0 &&
+                       ra.out_batch_stride % 4 == 0 && (((uintptr_t)ra.out | (uintptr_t)ra.partial) & 15) == 0 &&
+                       (outs / 4 + WG_THREADS - 1) / WG_THREADS < (1ll << 31);
+    if (rows4) {
+        splitk_reduce_rows4_kernel<<<dim3((unsigned)((outs / 4 + WG_THREADS - 1) / WG_THREADS), (unsigned)ra.batch), WG_THREADS, 0, stream>>>(ra);
+        return;
+    }
     if (outs * ra.batch <= 16384 && ra.nsplit >= 64)
         splitk_reduce_kernel<8><<<dim3((unsigned)((outs + 7) / 8), (unsigned)ra.batch), WG_THREADS, 0, stream>>>(ra);
     else
@@ -1040,6 +1074,13 @@ size_t gemm_workspace_bytes_wide(int64_t R, int64_t J, int64_t K, int batch, int
     return unsplit_bytes(R, J, K, batch, q_batches) + wide_workspace_bytes(R, J, K, batch);
 }
 
+size_t gemm_workspace_bytes_wide_planar(const GemmDesc &d)
+{
+    const size_t planar = wide_workspace_bytes_planar(d);
+    if (planar == 0 || !wide_shape_eligible(d.R, d.batch)) return 0;
+    return unsplit_bytes(d.R, d.J, d.K, d.batch, d.q.batches) + planar;
+}
+
 size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches)
 {
     const size_t need = gemm_workspace_bytes(R, J, K, batch, q_batches);
@@ -1151,8 +1192,15 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         // tables too wide for the LDS: the row-staged engine, if the workspace also holds the
         // transposed lane operand (else the global-gather variant below does the job, slowly)
         const Plan pq = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, false, WAVES_PER_SIMD);
-        if (workspace != nullptr && ((uintptr_t)workspace & 255) == 0 &&
-            workspace_bytes >= pq.total + wide_workspace_bytes(d.R, d.J, d.K, d.batch)) {
+        // convolution patches: from an im2col in the workspace if it holds one (KH x KW times the source:
+        // streamed once, the fastest), else from a zero-bordered channel-major copy of the source (its own
+        // size; every plane is re-read once per filter tap, about 25 % slower overall), else -- below --
+        // one global gather per product
+        const bool ws_ok = workspace != nullptr && ((uintptr_t)workspace & 255) == 0;
+        const bool im2col = ws_ok && workspace_bytes >= pq.total + wide_workspace_bytes(d.R, d.J, d.K, d.batch);
+        const size_t planar_need = im2col ? 0 : wide_workspace_bytes_planar(d);
+        const bool planar = ws_ok && planar_need > 0 && workspace_bytes >= pq.total + planar_need;
+        if (im2col || planar) {
             uint8_t *ws = static_cast<uint8_t *>(workspace);
             QArgs qa{};
             qa.q = d.q;
@@ -1161,7 +1209,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
             qa.qflags = reinterpret_cast<uint32_t *>(ws + pq.off_flags);
             qa.qdesc_out = reinterpret_cast<QDesc *>(ws + pq.off_qdesc);
             if (const int rc = launch_q_prepass(qa, d.q.batches, stream)) return rc;
-            return run_gemm_wide(lut, d, WideQ{qa.qw, qa.qflags, qa.qdesc_out, pq.Jp, pq.nchunks}, ws + pq.total, may_split, stream);
+            return run_gemm_wide(lut, d, WideQ{qa.qw, qa.qflags, qa.qdesc_out, pq.Jp, pq.nchunks}, ws + pq.total, planar, may_split, stream);
         }
     }
     const Plan pl = make_plan(d.R, d.J, d.K, d.batch, d.q.batches, may_split, waves64_of(d.p, d.K));

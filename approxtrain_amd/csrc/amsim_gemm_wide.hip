@@ -57,6 +57,7 @@ struct PTArgs {
 __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
 {
     __shared__ uint32_t tile[KC][PT_ROWS + 1];
+    __shared__ int4 rowinfo[PT_ROWS];  // patch sources: {element offset of the window origin, y origin, x origin, row inside R}
     const int64_t G = a.Rp / PT_ROWS;
     const int64_t g = blockIdx.x % G, ch = blockIdx.x / G;
     const int bz = blockIdx.y;
@@ -67,6 +68,42 @@ __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
     // (channels run fastest in both the image and the reduction index)
     const bool k_fast = a.p.kind == P_PATCH || (a.p.kind == P_DENSE && a.p.sk == 1 && a.p.sr != 1);
     SafeRange range;
+    if (a.p.kind == P_PATCH) {
+        // A thread's reduction index is the same for all its elements (lanes run along k): decomposed
+        // once; the rows' window origins once per workgroup, through LDS -- instead of four divisions
+        // per element.
+        if (tid < PT_ROWS) {
+            const int64_t r = g * PT_ROWS + tid;
+            int4 v = make_int4(0, 0, 0, 0);
+            if (r < a.R) {
+                const uint32_t r32 = (uint32_t)r, gw = (uint32_t)a.p.GW, gh = (uint32_t)a.p.GH;  // (fewer than 2^31 rows)
+                const int x = (int)(r32 % gw);
+                const uint32_t t = r32 / gw;
+                const int y = (int)(t % gh), b = (int)(t / gh);
+                const int vy0 = y * a.p.sy - a.p.pt, vx0 = x * a.p.sx - a.p.pl;
+                v = make_int4(((b * a.p.SH + vy0) * a.p.SW + vx0) * a.p.C, vy0, vx0, 1);
+            }
+            rowinfo[tid] = v;
+        }
+        __syncthreads();
+        const int kk = tid % KC;
+        const int64_t k = ch * KC + kk;
+        const uint32_t k32 = (uint32_t)k, c32 = (uint32_t)a.p.C;
+        const int c = (int)(k32 % c32), tap = (int)(k32 / c32);
+        const int fx = tap % a.p.KW, fy = tap / a.p.KW;
+        const int tapoff = (fy * a.p.SW + fx) * a.p.C + c;
+        const bool kvalid = k < a.K;
+#pragma unroll
+        for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
+            const int rl = tid / KC + (WG_THREADS / KC) * i;
+            const int4 ri = rowinfo[rl];
+            uint32_t raw = 0u;
+            if (kvalid && ri.w && (unsigned)(ri.y + fy) < (unsigned)a.p.SH && (unsigned)(ri.z + fx) < (unsigned)a.p.SW)
+                raw = f2u(pbase[ri.x + tapoff]);
+            range.add(raw);
+            tile[kk][rl] = raw;
+        }
+    } else {
 #pragma unroll
     for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
         const int e = tid + WG_THREADS * i;
@@ -77,6 +114,7 @@ __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
         const uint32_t raw = p_raw_bits(a.p, pbase, a.R, a.K, r, k);
         range.add(raw);
         tile[kk][rl] = raw;
+    }
     }
     // the tile's operand span: per wavefront by shuffles, across the four through LDS
     __shared__ uint32_t wave_range[WG_THREADS / 64][2];
@@ -170,13 +208,26 @@ struct WArgs {
     int nsplit;              // slices of the reduction (blockIdx.z), each a whole number of chunks
     int chunks_per_split;
     float *partial;          // nsplit > 1: [nsplit][batch][X * tile rows][Jp] partial sums instead of `out`
+    // PLANAR (convolution patches read from a channel-major copy of the source instead of an im2col):
+    // `pt` is [channel][pixel] with plane_elems pixels per channel, `pflags` [channel chunk][64-pixel group]
+    PDesc p;
+    int64_t plane_elems;     // B * ph * pw, rounded up to whole 64-pixel groups
+    int ph, pw;              // padded image extent: (GH - 1) * sy + KH rows, (GW - 1) * sx + KW columns
+    int cchunks;
 };
 
 // MPT: pairs of lane-mantissa values each thread stages per reduction step (2 at width 11: 2048 values
 // over 512 threads; 1 below, where the wavefronts past the row's end stage nothing).
 // RPT: rows per thread, 8 (4096 rows per workgroup: 1 byte of table row pulled per product) or 4 (2048
 // rows, 2 bytes per product: for problems that would otherwise leave compute units without a workgroup).
-template <int MPT, int RPT>
+// PLANAR: the lane operand of a convolution (forward / input gradient) is read from a channel-major,
+// zero-bordered copy of the source image, xT[c][b][py][px] with py = source row + pad_top and
+// px = source column + pad_left, instead of from an im2col in [k][row] order: element
+// (row (b, y, x), k (fy, fx, c)) is xT[c][(b * PH + y * sy + fy) * PW + x * sx + fx], so for one
+// reduction step all rows read one channel plane at a uniform shift -- consecutive rows read
+// consecutive words (stride sx), no window test, no vector instruction spent on addresses -- and the
+// copy is the size of the (padded) source, not KH * KW times it.
+template <int MPT, int RPT, bool PLANAR>
 __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
 {
     constexpr int TILE_ROWS = WIDE_THREADS * RPT;
@@ -211,7 +262,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     const uint32_t *ptile = a.pt + (size_t)bz * Kp * a.Rp + row0;  // [k][this workgroup's rows]
     const uint32_t voff = (uint32_t)tid * 4u;                        // this thread's byte offset in a run of dwords
     const rsrc_t lut_rsrc = make_rsrc(a.lut16);
-    const int64_t G = a.Rp / PT_ROWS;
+    const int64_t G = (PLANAR ? a.plane_elems : a.Rp) / PT_ROWS;  // 64-row (PLANAR: 64-pixel) groups per flag row
     const uint32_t *pfl = a.pflags + (size_t)bz * a.nchunks * G;
     uint32_t c256 = 256u;
     asm volatile("" : "+v"(c256));  // stays in a vector register (the factor instruction has one scalar port)
@@ -257,10 +308,51 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         }
     };
     uint32_t pc[RPT], pn[RPT];
-    auto load_p = [&](int k, uint32_t (&dst)[RPT]) {
-        const rsrc_t src = make_rsrc(ptile + (size_t)k * a.Rp);
+    // PLANAR: per row the byte offset of its window origin inside a channel plane; per reduction step
+    // (walked, k = (fy, fx, c) with the channel fastest) the channel and the tap.
+    uint32_t pixoff[PLANAR ? RPT : 1];
+    int w_c = 0, w_tap = 0, w_fx = 0, w_fy = 0;      // the step whose operands load_p fetches next
+    if (PLANAR) {
 #pragma unroll
-        for (int rr = 0; rr < RPT; ++rr) dst[rr] = load_u32(src, voff, rr * (WIDE_THREADS * 4));
+        for (int rr = 0; rr < RPT; ++rr) {
+            const int64_t r = row0 + rr * WIDE_THREADS + tid;
+            uint32_t off = 0u;  // (padding rows read the first pixel: their sums are never stored)
+            if (r < a.R) {
+                const uint32_t r32 = (uint32_t)r, gw = (uint32_t)a.p.GW, gh = (uint32_t)a.p.GH;  // (fewer than 2^31 rows)
+                const uint32_t x = r32 % gw, t = r32 / gw;
+                const uint32_t y = t % gh, b = t / gh;
+                off = ((b * (uint32_t)a.ph + y * (uint32_t)a.p.sy) * (uint32_t)a.pw + x * (uint32_t)a.p.sx) * 4u;
+            }
+            pixoff[rr] = off;
+        }
+        const uint32_t k0 = (uint32_t)kbeg, C = (uint32_t)a.p.C;
+        w_c = (int)(k0 % C);
+        w_tap = (int)(k0 / C);
+        w_fx = w_tap % a.p.KW;
+        w_fy = w_tap / a.p.KW;
+    }
+    // moves the walk on by one reduction step
+    auto walk_step = [&]() {
+        if (++w_c == a.p.C) {
+            w_c = 0;
+            ++w_tap;
+            if (++w_fx == a.p.KW) { w_fx = 0; ++w_fy; }
+        }
+    };
+    auto load_p = [&](int k, uint32_t (&dst)[RPT]) {
+        if constexpr (PLANAR) {
+            // reduction steps past the filter (the last chunk's padding) read nothing: a buffer of no
+            // records returns zero for every lane
+            const bool live = w_tap < a.p.KH * a.p.KW;
+            const rsrc_t src = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(a.pt), 0, live ? 0x7fffffff : 0, 0x00020000);
+            const uint32_t shift = live ? (uint32_t)((size_t)w_c * a.plane_elems + (size_t)(w_fy * a.pw + w_fx)) * 4u : 0u;
+#pragma unroll
+            for (int rr = 0; rr < RPT; ++rr) dst[rr] = load_u32(src, pixoff[rr], shift);
+        } else {
+            const rsrc_t src = make_rsrc(ptile + (size_t)k * a.Rp);
+#pragma unroll
+            for (int rr = 0; rr < RPT; ++rr) dst[rr] = load_u32(src, voff, rr * (WIDE_THREADS * 4));
+        }
     };
 
     fetch_rows(kbeg);
@@ -274,9 +366,25 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
     int tile_flagged = 0;
     for (int ch = ch_beg + tid; ch < ch_end; ch += WIDE_THREADS)
         tile_flagged |= (int)(a.qflags[qt_index * a.nchunks + ch] >> 31);
+    // PLANAR: the 64-pixel groups that the tile's rows can read at any tap, over every channel chunk
+    int64_t pg_lo = 0, pg_hi = -1;
+    if (PLANAR) {
+        auto pixel_of = [&](int64_t r) -> int64_t {
+            const uint32_t r32 = (uint32_t)r, gw = (uint32_t)a.p.GW, gh = (uint32_t)a.p.GH;
+            const int64_t x = r32 % gw, t = r32 / gw;
+            return ((t / gh) * a.ph + (t % gh) * a.p.sy) * a.pw + x * a.p.sx;
+        };
+        const int64_t last_row = min(row0 + TILE_ROWS, a.R) - 1;
+        pg_lo = pixel_of(row0) / PT_ROWS;
+        pg_hi = min(a.plane_elems - 1, pixel_of(last_row) + (int64_t)(a.p.KH - 1) * a.pw + (a.p.KW - 1)) / PT_ROWS;
+        const int64_t ngroups = pg_hi - pg_lo + 1;
+        for (int64_t i = tid; i < ngroups * a.cchunks; i += WIDE_THREADS)
+            tile_flagged |= (int)(a.pflags[(size_t)(i / ngroups) * G + pg_lo + i % ngroups] >> 31);
+    } else {
     for (int i = tid; i < (ch_end - ch_beg) * (TILE_ROWS / PT_ROWS); i += WIDE_THREADS)
         tile_flagged |= (int)(pfl[(size_t)(ch_beg + i / (TILE_ROWS / PT_ROWS)) * G + (size_t)bx * (TILE_ROWS / PT_ROWS) +
                                   i % (TILE_ROWS / PT_ROWS)] >> 31);
+    }
     tile_flagged = __syncthreads_or(tile_flagged);
 
     // one stage: the rows of stage k + 1 are fetched while stage k gathers from `cur`, and regrouped
@@ -286,6 +394,7 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
         // (the last stage fetches its own rows and operands once more instead of branching: a
         // straight-line stage keeps the compiler from sinking one stage's FMAs into the next)
         const int kn = min(k + 1, kend - 1);
+        if (PLANAR && k + 1 < kend) walk_step();
         if constexpr (!EXACT) {
             uint32_t qt[WIDE_TN];
 #pragma unroll
@@ -343,11 +452,37 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
             stage(std::false_type{}, k + 1, rows_b, rows_a);
         }
     } else {
+        // PLANAR: one span for everything the tile can read (every channel chunk, every pixel group in
+        // reach): coarser than a span per chunk, which only matters to inputs that hold values outside
+        // the fast product's range in the first place
+        uint32_t planar_span = 0u, planar_quick = 0u;
+        if (PLANAR) {
+            SafeRange join;
+            uint32_t quick = 0u, hard = 0u;
+            const int64_t ngroups = pg_hi - pg_lo + 1;
+            for (int64_t i = lane; i < ngroups * a.cchunks; i += 64) {
+                const uint32_t pf = a.pflags[(size_t)(i / ngroups) * G + pg_lo + i % ngroups];
+                quick |= pf & SPAN_QUICK_FAIL;
+                hard |= pf & SPAN_HARD;
+                if ((pf & 0xffffu) != 0xff00u) {  // (not an all-zero group)
+                    join.tmax = max(join.tmax, (pf & 255u) << 24);
+                    join.tmin = min(join.tmin, ((pf >> 8) & 255u) << 24);
+                }
+            }
+            join = wave_union(join);
+            const uint32_t emax = join.tmax >> 24, emin = join.tmin == 0xffffffffu ? 255u : join.tmin >> 24;
+            planar_span = (__any(hard != 0u) ? SPAN_HARD : 0u) | (emin << 8) | emax;
+            planar_quick = __any(quick != 0u) ? SPAN_QUICK_FAIL : 0u;
+        }
         for (int ch = ch_beg; ch < ch_end; ++ch) {
             // spans of the tile's 64-row groups (one per lane: TILE_ROWS / 64 <= 64), joined; the chunk is
             // slow only if a quick test failed AND the joined span is not compatible with the uniform operand's
             SafeRange join;
             uint32_t quick = qfl[ch] & SPAN_QUICK_FAIL, hard = 0u;
+            bool unsafe;
+            if (PLANAR) {
+                unsafe = ((quick | planar_quick) != 0u) && !spans_compatible(planar_span, qfl[ch]);
+            } else {
             if (lane < TILE_ROWS / PT_ROWS) {
                 const uint32_t pf = pfl[(size_t)ch * G + (size_t)bx * (TILE_ROWS / PT_ROWS) + lane];
                 quick |= pf & SPAN_QUICK_FAIL;
@@ -357,12 +492,13 @@ __global__ __launch_bounds__(WIDE_THREADS, 4) void lutgemm_wide_kernel(WArgs a)
                     join.tmin = ((pf >> 8) & 255u) << 24;
                 }
             }
-            bool unsafe = __any(quick != 0u) != 0;
+            unsafe = __any(quick != 0u) != 0;
             if (unsafe) {
                 join = wave_union(join);
                 const uint32_t emax = join.tmax >> 24, emin = join.tmin == 0xffffffffu ? 255u : join.tmin >> 24;
                 const uint32_t pspan = (__any(hard != 0u) ? SPAN_HARD : 0u) | (emin << 8) | emax;
                 unsafe = !spans_compatible(pspan, qfl[ch]);
+            }
             }
             if (!unsafe) {
 #pragma unroll 1
@@ -435,7 +571,10 @@ struct WidePlan {
     int64_t Rp, X, strips, nchunks;
     size_t pt_bytes, flag_bytes, partial_bytes;
 };
-WidePlan wide_plan(int64_t R, int64_t J, int64_t K, int batch, bool may_split, int cus)
+// planar_pixels > 0: the lane operand is a convolution's source read from its channel-major copy
+// (planar_channels planes of that many pixels) instead of an im2col of K x Rp words
+WidePlan wide_plan(int64_t R, int64_t J, int64_t K, int batch, bool may_split, int cus, int64_t planar_pixels = 0,
+                   int planar_channels = 0)
 {
     WidePlan pl{};
     pl.Rp = padded_rows(R);
@@ -443,32 +582,85 @@ WidePlan wide_plan(int64_t R, int64_t J, int64_t K, int batch, bool may_split, i
     pl.strips = (J + QT - 1) / QT * (QT / WIDE_TN);
     const int64_t slots = 2 * (int64_t)cus;
     pl.tile_rows = (int)std::min<int64_t>(pl.Rp, WIDE_TILE_ROWS);
-    // half-height tiles when full-height ones would leave slots empty
-    if (pl.tile_rows == WIDE_TILE_ROWS && (pl.Rp / WIDE_TILE_ROWS) * pl.strips * batch < slots) pl.tile_rows = WIDE_TILE_ROWS / 2;
-    pl.X = (R + pl.tile_rows - 1) / pl.tile_rows;
-    const int64_t tiles = pl.X * pl.strips * batch;
     pl.nsplit = 1;
     pl.chunks_per_split = (int)pl.nchunks;
-    // (slices of at least 4 chunks = 128 stages, a few hundred microseconds: shorter ones would not
-    // pay for their partial sums and the reduction launch)
-    if (may_split && 2 * tiles <= slots && pl.nchunks >= 16) {
+    // Problems taller than one tile: full-height tiles (1 byte of table row pulled per product, + 0.5 of
+    // lane operand) or half-height ones (2 + 0.5), and the reduction whole or in slices of at least 4
+    // chunks (128 stages: shorter ones do not pay for their partial sums).  What bounds the kernel is the
+    // bytes pulled from L2, shared by the resident workgroups (two per compute unit; a workgroup with a
+    // compute unit to itself gets about 1.5 shares), in rounds of as many workgroups as fit; slices add
+    // the write + re-read of their partial sums and the reduction launch.  The cheapest combination wins.
+    const bool tall = pl.tile_rows == WIDE_TILE_ROWS;
+    if (tall) {
+        const double pull = 13.5e12, partial_rate = 3.0e12, launch_s = 8.0e-6;
+        const int64_t Jp = pl.strips * WIDE_TN;
+        double best = 0;
+        for (int rows : {WIDE_TILE_ROWS, WIDE_TILE_ROWS / 2}) {
+            const int64_t X = (R + rows - 1) / rows, tiles = X * pl.strips * batch;
+            const double bytes_per_product = (double)WIDE_TILE_ROWS / rows + 0.5;
+            const int64_t smax = may_split ? std::max<int64_t>(1, std::min<int64_t>(pl.nchunks / 4, 65535)) : 1;
+            for (int64_t want = 1; want <= smax; ++want) {
+                const int64_t cps = (pl.nchunks + want - 1) / want, ns = (pl.nchunks + cps - 1) / cps;
+                if (ns != want) continue;
+                const int64_t wgs = tiles * ns, rounds = (wgs + slots - 1) / slots;
+                const double share = pull / (double)std::max<int64_t>(std::min(wgs, slots), slots * 2 / 3);
+                double t = (double)rounds * cps * KC * rows * WIDE_TN * bytes_per_product / share;
+                if (ns > 1) t += 2.0 * ns * (double)batch * X * rows * Jp * sizeof(float) / partial_rate + launch_s;
+                if (best == 0 || t < best) { best = t; pl.tile_rows = rows; pl.nsplit = (int)ns; pl.chunks_per_split = (int)cps; }
+            }
+        }
+    }
+    pl.X = (R + pl.tile_rows - 1) / pl.tile_rows;
+    const int64_t tiles = pl.X * pl.strips * batch;
+    // one short tile (filter gradients: a few hundred to a few thousand rows, a very long reduction):
+    // slices when the tiles alone leave half or more of the slots empty
+    if (!tall && may_split && 2 * tiles <= slots && pl.nchunks >= 16) {
         const int64_t want = std::min<int64_t>(pl.nchunks / 4, std::min<int64_t>((slots + tiles - 1) / tiles, 65535));
         pl.chunks_per_split = (int)((pl.nchunks + want - 1) / want);
         pl.nsplit = (int)((pl.nchunks + pl.chunks_per_split - 1) / pl.chunks_per_split);
     }
     pl.pt_bytes = align256((size_t)batch * pl.nchunks * KC * pl.Rp * sizeof(uint32_t));
     pl.flag_bytes = align256((size_t)batch * pl.nchunks * (pl.Rp / PT_ROWS) * sizeof(uint32_t));
+    if (planar_pixels > 0) {
+        const int64_t pixp = (planar_pixels + PT_ROWS - 1) / PT_ROWS * PT_ROWS, cch = (planar_channels + KC - 1) / KC;
+        pl.pt_bytes = align256((size_t)cch * KC * pixp * sizeof(uint32_t));
+        pl.flag_bytes = align256((size_t)cch * (pixp / PT_ROWS) * sizeof(uint32_t));
+    }
     const int64_t Jp = pl.strips * WIDE_TN;
     pl.partial_bytes = pl.nsplit > 1 ? align256((size_t)pl.nsplit * batch * pl.X * pl.tile_rows * Jp * sizeof(float)) : 0;
     return pl;
 }
 
 template <int RPT>
-void launch_wide(const WArgs &wa, dim3 grid, int m, hipStream_t stream)
+void launch_wide(const WArgs &wa, dim3 grid, int m, bool planar, hipStream_t stream)
 {
-    if (m >= 11) lutgemm_wide_kernel<2, RPT><<<grid, WIDE_THREADS, 0, stream>>>(wa);
-    else lutgemm_wide_kernel<1, RPT><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+    if (planar) {
+        if (m >= 11) lutgemm_wide_kernel<2, RPT, true><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        else lutgemm_wide_kernel<1, RPT, true><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+    } else {
+        if (m >= 11) lutgemm_wide_kernel<2, RPT, false><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+        else lutgemm_wide_kernel<1, RPT, false><<<grid, WIDE_THREADS, 0, stream>>>(wa);
+    }
 }
+
+// A convolution's patches can be read from a channel-major, zero-bordered copy of its source when
+// the whole copy stays below 2^31 bytes (one buffer resource addresses it) and the batch is folded
+// into the rows (the convolution entry points do that).  Returns the pixels of one channel plane, 0 if
+// the form does not apply.
+struct Planar { int ph, pw; int64_t pixels; };
+Planar planar_of(const GemmDesc &d)
+{
+    Planar pn{0, 0, 0};
+    if (d.p.kind != P_PATCH || d.batch != 1 || d.p.KH < 1 || d.p.KW < 1 || d.p.GH < 1 || d.p.GW < 1 || d.p.C < 1) return pn;
+    if (d.K != (int64_t)d.p.KH * d.p.KW * d.p.C) return pn;
+    const int64_t ph = (int64_t)(d.p.GH - 1) * d.p.sy + d.p.KH, pw = (int64_t)(d.p.GW - 1) * d.p.sx + d.p.KW;
+    const int64_t pixels = (int64_t)d.p.B * ph * pw, pixp = (pixels + PT_ROWS - 1) / PT_ROWS * PT_ROWS;
+    const int64_t cp = (int64_t)((d.p.C + KC - 1) / KC) * KC;
+    if (ph >= (1 << 20) || pw >= (1 << 20) || pixp * cp * 4 >= (1ll << 31) - 4096) return pn;
+    pn.ph = (int)ph; pn.pw = (int)pw; pn.pixels = pixels;
+    return pn;
+}
+inline int64_t planar_pixels(const GemmDesc &d) { return planar_of(d).pixels; }
 
 }  // namespace
 
@@ -499,17 +691,45 @@ size_t wide_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch)
     return need;
 }
 
-int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, bool may_split, hipStream_t stream)
+size_t wide_workspace_bytes_planar(const GemmDesc &d)
 {
-    const WidePlan pl = wide_plan(d.R, d.J, d.K, d.batch, may_split, device_compute_units());
+    const int64_t pixels = planar_pixels(d);
+    if (pixels == 0) return 0;
+    size_t need = 0;
+    for (int cus : {device_compute_units(), 256, 304})
+        for (bool split : {false, true}) {
+            const WidePlan pl = wide_plan(d.R, d.J, d.K, d.batch, split, cus, pixels, d.p.C);
+            need = std::max(need, pl.pt_bytes + pl.flag_bytes + pl.partial_bytes);
+        }
+    return need;
+}
+
+int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, bool planar, bool may_split, hipStream_t stream)
+{
+    const int64_t pixels = planar ? planar_pixels(d) : 0;
+    const WidePlan pl = wide_plan(d.R, d.J, d.K, d.batch, may_split, device_compute_units(), pixels, d.p.C);
     const int64_t Rp = pl.Rp;
-    const int64_t G = Rp / PT_ROWS;
     uint8_t *ws = static_cast<uint8_t *>(wide_ws);
     PTArgs pa{};
-    pa.p = d.p; pa.R = d.R; pa.K = d.K; pa.Rp = Rp; pa.nchunks = q.nchunks;
     pa.pt = reinterpret_cast<uint32_t *>(ws);
     pa.pflags = reinterpret_cast<uint32_t *>(ws + pl.pt_bytes);
-    const int64_t pwgs = G * q.nchunks;
+    int64_t pwgs;
+    const Planar pn = planar_of(d);
+    if (pixels > 0) {
+        // the zero-bordered source as a [padded pixel][channel] matrix, transposed into channel planes:
+        // a 1x1 "convolution" over the padded extent reads source pixel (py - pad_top, px - pad_left), zero outside
+        pa.p = PDesc{};
+        pa.p.kind = P_PATCH; pa.p.base = d.p.base;
+        pa.p.B = d.p.B; pa.p.GH = pn.ph; pa.p.GW = pn.pw; pa.p.KH = 1; pa.p.KW = 1; pa.p.C = d.p.C;
+        pa.p.sy = 1; pa.p.sx = 1; pa.p.pt = d.p.pt; pa.p.pl = d.p.pl; pa.p.SH = d.p.SH; pa.p.SW = d.p.SW;
+        pa.R = pixels; pa.K = d.p.C;
+        pa.Rp = (pixels + PT_ROWS - 1) / PT_ROWS * PT_ROWS;
+        pa.nchunks = (d.p.C + KC - 1) / KC;
+        pwgs = (pa.Rp / PT_ROWS) * pa.nchunks;
+    } else {
+        pa.p = d.p; pa.R = d.R; pa.K = d.K; pa.Rp = Rp; pa.nchunks = q.nchunks;
+        pwgs = (Rp / PT_ROWS) * q.nchunks;
+    }
     if (pwgs >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "lane operand exceeds the grid limit");
     p_linear_kernel<<<dim3((unsigned)pwgs, (unsigned)d.batch), WG_THREADS, 0, stream>>>(pa);
     AMSIM_HIP_CHECK(hipGetLastError());
@@ -530,13 +750,17 @@ int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_
     wa.nsplit = pl.nsplit;
     wa.chunks_per_split = pl.chunks_per_split;
     wa.partial = reinterpret_cast<float *>(ws + pl.pt_bytes + pl.flag_bytes);
+    wa.p = d.p;
+    wa.plane_elems = pixels > 0 ? pa.Rp : 0;
+    wa.ph = pn.ph; wa.pw = pn.pw;
+    wa.cchunks = pixels > 0 ? pa.nchunks : 0;
     const int64_t total = (int64_t)wa.X * wa.Y;
     if (total >= (1ll << 31)) return fail(AMSIM_ERR_UNSUPPORTED, "workgroup count exceeds the grid limit");
     const dim3 grid((unsigned)total, (unsigned)d.batch, (unsigned)pl.nsplit);
     switch (pl.tile_rows / WIDE_THREADS) {
-    case 8: launch_wide<8>(wa, grid, lut.m, stream); break;
-    case 4: launch_wide<4>(wa, grid, lut.m, stream); break;
-    default: launch_wide<2>(wa, grid, lut.m, stream); break;
+    case 8: launch_wide<8>(wa, grid, lut.m, pixels > 0, stream); break;
+    case 4: launch_wide<4>(wa, grid, lut.m, pixels > 0, stream); break;
+    default: launch_wide<2>(wa, grid, lut.m, pixels > 0, stream); break;
     }
     AMSIM_HIP_CHECK(hipGetLastError());
     if (pl.nsplit > 1) {

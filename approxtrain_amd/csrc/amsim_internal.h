@@ -135,12 +135,19 @@ struct WideQ {
 bool wide_shape_eligible(int64_t R, int batch);
 bool wide_eligible(int m, const GemmDesc &d, bool may_split);
 size_t wide_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch);
-int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, bool may_split, hipStream_t stream);
+// what the engine needs on top of the unsplit plan when a convolution's patches are read from a
+// channel-major copy of the source (its own size) instead of an im2col; 0 when that form does not apply
+size_t wide_workspace_bytes_planar(const GemmDesc &d);
+// planar: wide_ws holds wide_workspace_bytes_planar(d), else wide_workspace_bytes(...)
+int run_gemm_wide(const Lut &lut, const GemmDesc &d, const WideQ &q, void *wide_ws, bool planar, bool may_split, hipStream_t stream);
 // workspace that serves a dense problem with any table: the larger of gemm_workspace_bytes and
 // what the row-staged engine needs
 size_t gemm_workspace_bytes_any_lut(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
 // what the row-staged engine needs for a problem in all (unsplit plan + transposed lane operand)
 size_t gemm_workspace_bytes_wide(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
+// ... and with a convolution's patches read from a channel-major copy of the source instead of an
+// im2col (0 when that form does not apply)
+size_t gemm_workspace_bytes_wide_planar(const GemmDesc &d);
 
 // ---- the direct engine for small problems (one launch, operands read where they lie) ----------
 // Tables that fit the LDS only; which problems it takes is decided in direct_eligible().

@@ -14,7 +14,7 @@ layer, LeNet-5 convolutions, the 4096^3 GEMM sweep over ten tables, the
 attention block, and every convolution of ResNet-50's bottleneck stages) under "configs", and the CPU oracle timed on a bounded sample
 of the headline workload on the host cores.
 
-`--only NAME` runs one workload alone (headline, cfg1, cfg2, cfg4, cfg4-m11,
+`--only NAME` runs one workload alone (headline, cfg1, cfg2, cfg3-m11, cfg4, cfg4-m11,
 cfg5, resnet50) without micro-kernels or CPU baseline: the form the profiler runs.
 """
 import argparse
@@ -208,10 +208,26 @@ def cpu_baseline(x, w, dy):
 
 # ---- the other benchmark configurations ---------------------------------------------------------
 
-def _entry(macs, ms, roof_gmacs):
+def _entry(macs, ms, roof_gmacs, lds_roof_gmacs=None, min_bytes_per_product=None, pull_bytes_per_s=None):
+    """lds_roof_gmacs / min_bytes_per_product (width-11 entries): the rate also as a fraction of the
+    roof of tables that fit the LDS, and against what the problem itself allows -- the table-row bytes
+    a tile of the problem's own row count must pull from L2 per product (a 4 KB row per column and
+    reduction step serves at most min(rows, 4096) products) plus 0.5 byte of lane operand -- at the
+    measured pull rate: a bound set by the problem, not by this engine's choice of tile."""
     g = macs / (ms * 1e-3) / 1e9
-    return {"macs": int(macs), "device_ms": round(ms, 4), "gmacs": round(g, 1),
-            "roof_frac": round(g / roof_gmacs, 4) if roof_gmacs else None}
+    e = {"macs": int(macs), "device_ms": round(ms, 4), "gmacs": round(g, 1),
+         "roof_frac": round(g / roof_gmacs, 4) if roof_gmacs else None}
+    if lds_roof_gmacs:
+        e["frac_of_lds_table_roof"] = round(g / lds_roof_gmacs, 4)
+    if min_bytes_per_product and pull_bytes_per_s:
+        e["min_l2_bytes_per_product"] = round(min_bytes_per_product, 3)
+        e["frac_of_l2_pull_bound_at_min_bytes"] = round(g * 1e9 * min_bytes_per_product / pull_bytes_per_s, 4)
+    return e
+
+
+def wide_min_bytes_per_product(rows):
+    """Bytes a width-11 problem with `rows` rows over the lanes must pull from L2 per product."""
+    return 4096.0 / min(max(rows, 1), 4096) + 0.5
 
 
 def glorot(rng, shape, fan_in, fan_out):
@@ -254,7 +270,24 @@ def run_cfg2(roof):
     return out
 
 
-def run_cfg4(roof, wide_roof, tables=None):
+def run_cfg3_wide(roof, wide_roof, pull):
+    """The headline layer (cfg3) with the width-11 table MBM_11: forward, grad-input, grad-filter on the
+    row-staged engine (the forward / grad-input patches from an im2col in the workspace, the filter
+    gradient's 576 filter elements over the lanes)."""
+    import torch
+    from approxtrain_amd import functors
+    lut = make_lut("MBM", 11)
+    _, _, _, (xd, wd, dyd) = synthetic("cuda")
+    passes = (("fwd", 32 * 56 * 56, lambda: functors.convam(lut, xd, wd, (1, 1), "SAME")),
+              ("grad_input", 32 * 56 * 56, lambda: functors.convam_input_grad(lut, XS, wd, dyd, (1, 1), "SAME")),
+              ("grad_filter", 3 * 3 * 64, lambda: functors.convam_filter_grad(lut, xd, WS, dyd, (1, 1), "SAME")))
+    out = {name: _entry(MACS_PER_PASS, device_ms(fn), wide_roof, roof, wide_min_bytes_per_product(rows), pull)
+           for name, rows, fn in passes}
+    lut.close()
+    return out
+
+
+def run_cfg4(roof, wide_roof, tables=None, pull=None):
     """MatMulAM 4096^3 sweep: C = A.B, dA = dC.B^T, dB = A^T.dC with N(0,1) operands, for MBM and
     MIT at mantissa widths 1, 3, 5, 7 (table in LDS) and 11 (16-bit table in device memory, rows
     staged through LDS).  The width-11 tables come from the generator's closed-form rules: no
@@ -271,9 +304,10 @@ def run_cfg4(roof, wide_roof, tables=None):
                 continue
             lut = make_lut(kind, m)
             r = wide_roof if m > 7 else roof
-            e = {"C=A.B": _entry(n ** 3, device_ms(lambda: functors.gemm(lut, A, B)), r),
-                 "dA=dC.Bt": _entry(n ** 3, device_ms(lambda: functors.gemm(lut, dC, B, trans_b=True)), r),
-                 "dB=At.dC": _entry(n ** 3, device_ms(lambda: functors.gemm(lut, A, dC, trans_a=True)), r)}
+            extra = (roof, wide_min_bytes_per_product(n), pull) if m > 7 else ()
+            e = {"C=A.B": _entry(n ** 3, device_ms(lambda: functors.gemm(lut, A, B)), r, *extra),
+                 "dA=dC.Bt": _entry(n ** 3, device_ms(lambda: functors.gemm(lut, dC, B, trans_b=True)), r, *extra),
+                 "dB=At.dC": _entry(n ** 3, device_ms(lambda: functors.gemm(lut, A, dC, trans_a=True)), r, *extra)}
             out["%s_%d" % (kind, m)] = e
             lut.close()
     return out
@@ -398,7 +432,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="headline workload only")
-    ap.add_argument("--only", default=None, help="run one workload alone: headline, cfg1, cfg2, cfg4, cfg4-m11, cfg5, resnet50")
+    ap.add_argument("--only", default=None, help="run one workload alone: headline, cfg1, cfg2, cfg3-m11, cfg4, cfg4-m11, cfg5, resnet50")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -416,6 +450,7 @@ def main():
 
     if args.only and args.only != "headline":
         runners = {"cfg1": lambda: run_cfg1(None), "cfg2": lambda: run_cfg2(None), "cfg4": lambda: run_cfg4(None, None),
+                   "cfg3-m11": lambda: run_cfg3_wide(None, None, None),
                    "cfg4-m11": lambda: run_cfg4(None, None, tables={("MBM", 11), ("MIT", 11)}), "cfg5": lambda: run_cfg5(None),
                    "resnet50": lambda: run_resnet50(None)}
         if args.only not in runners:
@@ -477,6 +512,7 @@ def main():
         "lds_16_byte_scattered_reads": peaks["wide_lds_b128_scattered_products_per_s"] / 1e9,
     }
     wide_peak = min(wide_bounds.values())
+    wide_pull = max(peaks["wide_row_pull_bytes_per_s"], peaks["wide_row_pull_to_registers_bytes_per_s"])
     clock = clocks.get("valu_mix", SPEC_CLOCK_HZ)
     # dominant kernel: the patch-gather LUT GEMM of the forward pass (grad-input runs the same kernel)
     achieved = MACS_PER_PASS / (pass_ms["fwd"] * 1e-3) / 1e9
@@ -531,8 +567,10 @@ def main():
                     "enqueue time, from the replay of a captured graph of 40 calls), MACs as counted for the headline, roof_frac against "
                     "roofline.peak (tables in LDS) or roofline.wide_table_peak_gmacs (width 11: the lowest of "
                     "roofline.wide_table_bounds_gmacs -- bytes pulled in from L2 at 1.5 per product, the factor + FMA "
-                    "instruction pair, scattered 16-byte LDS reads)",
-            "cfg1": run_cfg1(peak), "cfg2": run_cfg2(peak), "cfg4": run_cfg4(peak, wide_peak), "cfg5": run_cfg5(peak),
+                    "instruction pair, scattered 16-byte LDS reads); width-11 entries also carry their fraction of the LDS-table "
+                    "roof and of the L2 pull bound at the bytes per product the problem's own row count requires",
+            "cfg1": run_cfg1(peak), "cfg2": run_cfg2(peak), "cfg3_MBM_11": run_cfg3_wide(peak, wide_peak, wide_pull),
+            "cfg4": run_cfg4(peak, wide_peak, pull=wide_pull), "cfg5": run_cfg5(peak),
             "resnet50_convolutions_batch32": run_resnet50(peak),
         }
     if not args.no_cpu_baseline:

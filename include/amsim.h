@@ -142,10 +142,16 @@ int amsim_convam_f32(amsim_lut_t lut, const float *input_data, float *output_dat
 /* The query for a given table.  For tables of up to 7 mantissa bits it equals the one above.  For
  * wider tables (8..11 bits) it adds what the row-staged engine needs -- an im2col of the input, the
  * temporary the reference also allocates (convam.cc:518-546) -- so that the call runs on that engine
- * (about 10x faster) instead of one global gather per product; a call given only the smaller amount
- * still runs, on the slow path. */
+ * at its best (the im2col is streamed once).  A call given less still runs: with at least the "lean"
+ * amount below, on the same engine from a zero-bordered channel-major copy of the input (the size
+ * of the input instead of filter_rows x filter_cols times it; about 25 % slower, every channel plane
+ * being re-read once per filter tap); with only the table-agnostic amount, by one global gather per
+ * product (about 10x slower). */
 size_t amsim_convam_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols, int out_depth,
                                         int filter_rows, int filter_cols, int in_depth);
+size_t amsim_convam_lean_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows, int out_cols, int out_depth,
+                                             int filter_rows, int filter_cols, int in_depth, int stride_rows,
+                                             int stride_cols);
 
 /* amsim_convam_f32 for callers that cannot allocate device memory or bring a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
@@ -154,8 +160,12 @@ size_t amsim_convam_workspace_bytes_for(amsim_lut_t lut, int batch, int out_rows
  * device image -- every GPU the library runs on holds it from the first call until the process
  * ends -- and calls no hipMalloc, hipFree or other allocating routine.  Problems whose
  * amsim_convam_workspace_bytes exceeds that size are refused with AMSIM_ERR_UNSUPPORTED.
- * Results are bit-identical to amsim_convam_f32 on the same inputs.  All calls on one GPU share
- * the one buffer: calls that may overlap there (different streams or threads) race; issue them
+ * Results are bit-identical to amsim_convam_f32 on the same inputs when that call is given a
+ * workspace of AMSIM_NOALLOC_SCRATCH_BYTES (for tables of up to 7 mantissa bits: any workspace its
+ * query returns; wider tables pick their engine by the workspace they are given, and engines
+ * differ in how they round split reductions).  The first call on a device also looks the buffer's
+ * address up (hipGetSymbolAddress): make one call outside a graph capture first.  All calls on one
+ * GPU share the one buffer: calls that may overlap there (different streams or threads) race; issue them
  * on one stream, or order them with events.  Nothing in the buffer needs to start at zero (each
  * call writes what it later reads). */
 #define AMSIM_NOALLOC_SCRATCH_BYTES ((size_t)32 << 20)

@@ -173,6 +173,72 @@ def test_convolution_forward_and_input_gradient_on_row_staged_engine(luts, kind,
     assert np.array_equal(dx.view(np.uint32), want_dx.view(np.uint32))
 
 
+@pytest.mark.parametrize("kind,m", [("MBM", 11), ("MIT", 8)])
+@pytest.mark.parametrize("shape", [((2, 24, 26, 8), (3, 3, 8, 20), (1, 1), "SAME"),
+                                   ((1, 40, 40, 3), (5, 4, 3, 7), (1, 1), "VALID"),
+                                   ((3, 30, 30, 16), (3, 3, 16, 12), (2, 2), "SAME"),
+                                   ((2, 33, 31, 40), (2, 3, 40, 9), (2, 1), "VALID"),
+                                   ((9, 20, 20, 64), (3, 3, 64, 24), (1, 1), "SAME")])   # several row tiles, sliced reduction
+def test_convolution_forward_from_the_channel_major_copy(luts, kind, m, shape):
+    """The lean workspace tier: given the amount amsim_convam_lean_workspace_bytes_for returns --
+    room for a zero-bordered channel-major copy of the input, not for an im2col -- the forward
+    pass runs on the row-staged engine from that copy.  Bit-equal to the oracle with reductions
+    kept whole, within 1e-5 * sum|products| with slices; a special value in the input takes the
+    full-domain path of the tiles that can reach it."""
+    import ctypes as C
+    import torch
+    import approxtrain_amd
+    from approxtrain_amd._lib import check, conv_geometry
+    from tests.gpu_util import assert_close_sum_abs
+    from tests.util import torch_conv_reference
+    from approxtrain_amd import ApproxMulLut
+    lib = approxtrain_amd.load_library()
+    _, img = luts(kind, m)
+    lut = ApproxMulLut.from_entries(_legacy(img), m)  # a handle of this test's own: it changes the split mode
+    assert lib.amsim_lut_set_split_k(lut.handle, 1) == 0
+    xs, ws, st, padding = shape
+    rng = np.random.default_rng(m * 10 + xs[1] + ws[1])
+    x = rng.standard_normal(xs).astype(np.float32)
+    x[rng.random(xs) < 0.3] = 0.0
+    w = rng.standard_normal(ws).astype(np.float32)
+    n, h, wd, c = xs
+    kh, kw, _, oc = ws
+    oh, pt = conv_geometry(h, kh, st[0], padding)
+    ow, pl = conv_geometry(wd, kw, st[1], padding)
+    lean = lib.amsim_convam_lean_workspace_bytes_for(lut.handle, n, oh, ow, oc, kh, kw, c, st[0], st[1])
+    full = lib.amsim_convam_workspace_bytes_for(lut.handle, n, oh, ow, oc, kh, kw, c)
+    assert lib.amsim_convam_workspace_bytes(n, oh, ow, oc, kh, kw, c) <= lean
+    if kh * kw >= 4:
+        assert lean < full, "the copy must be smaller than the im2col"
+    ws_t = torch.empty(lean + 256, dtype=torch.uint8, device="cuda")
+    wsp = ws_t.data_ptr() + (-ws_t.data_ptr()) % 256
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(xa):
+        xd, wdv = dev(xa), dev(w)
+        out = torch.full((n, oh, ow, oc), float("nan"), dtype=torch.float32, device="cuda")
+        check(lib.amsim_convam_f32(lut.handle, C.c_void_p(xd.data_ptr()), C.c_void_p(out.data_ptr()), n, oh, ow, oc, st[1], st[0],
+                                   pl, pt, kh, kw, c, wd, h, C.c_void_p(wdv.data_ptr()), C.c_void_p(wsp), lean, stream))
+        torch.cuda.synchronize()
+        return host(out)
+
+    want = cpu.conv2d_fwd(img, m, x, w, st, padding)
+    s_y, _, _ = torch_conv_reference(np.abs(x), np.abs(w), None, st, padding)
+    assert_close_sum_abs(run(x), want, s_y, 1e-5)
+    assert lib.amsim_lut_set_split_k(lut.handle, 0) == 0
+    assert np.array_equal(run(x).view(np.uint32), want.view(np.uint32))
+    # special values: an infinity, a NaN, a subnormal and a huge value somewhere in the image
+    xsp = x.copy()
+    flat = xsp.reshape(-1)
+    pos = rng.choice(flat.size, 4, replace=False)
+    flat[pos] = np.array([np.inf, np.nan, 1e-41, 3e38], np.float32)
+    want_sp = cpu.conv2d_fwd(img, m, xsp, w, st, padding)
+    got_sp = run(xsp)
+    from tests.util import same_bits_or_both_nan
+    assert same_bits_or_both_nan(got_sp, want_sp).all()
+    lut.close()
+
+
 def test_table_aware_convolution_query_adds_the_staged_operand_only_for_wide_tables(luts):
     import approxtrain_amd
     from approxtrain_amd import ApproxMulLut
