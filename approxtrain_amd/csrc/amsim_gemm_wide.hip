@@ -103,6 +103,42 @@ __global__ __launch_bounds__(WG_THREADS) void p_linear_kernel(PTArgs a)
             range.add(raw);
             tile[kk][rl] = raw;
         }
+    } else if (a.p.kind == P_GF) {
+        // Filter gradients: lanes run along the rows (filter elements; the channel is the contiguous
+        // direction of the source), so a thread's row is the same for all its elements: decomposed once;
+        // the chunk's 32 pixels once per workgroup, through LDS.
+        static_assert(KC <= PT_ROWS, "the pixel bookkeeping reuses the row bookkeeping's LDS");
+        if (tid < KC) {
+            const int64_t k = ch * KC + tid;
+            int4 v = make_int4(0, 0, 0, 0);
+            if (k < a.K) {
+                const uint32_t k32 = (uint32_t)k, gw = (uint32_t)a.p.GW, gh = (uint32_t)a.p.GH;  // (the reduction is shorter than 2^31)
+                const int x = (int)(k32 % gw);
+                const uint32_t t = k32 / gw;
+                const int y = (int)(t % gh), b = (int)(t / gh);
+                const int iy0 = y * a.p.sy - a.p.pt, ix0 = x * a.p.sx - a.p.pl;
+                v = make_int4(((b * a.p.SH + iy0) * a.p.SW + ix0) * a.p.C, iy0, ix0, 1);
+            }
+            rowinfo[tid] = v;
+        }
+        __syncthreads();
+        const int rl = tid % PT_ROWS;
+        const int64_t r = g * PT_ROWS + rl;
+        const uint32_t r32 = (uint32_t)r, c32 = (uint32_t)a.p.C;
+        const int c = (int)(r32 % c32), tap = (int)(r32 / c32);
+        const int fx = tap % a.p.KW, fy = tap / a.p.KW;
+        const int tapoff = (fy * a.p.SW + fx) * a.p.C + c;
+        const bool rvalid = r < a.R;
+#pragma unroll
+        for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
+            const int kk = tid / PT_ROWS + (WG_THREADS / PT_ROWS) * i;
+            const int4 ki = rowinfo[kk];
+            uint32_t raw = 0u;
+            if (rvalid && ki.w && (unsigned)(ki.y + fy) < (unsigned)a.p.SH && (unsigned)(ki.z + fx) < (unsigned)a.p.SW)
+                raw = f2u(pbase[ki.x + tapoff]);
+            range.add(raw);
+            tile[kk][rl] = raw;
+        }
     } else {
 #pragma unroll
     for (int i = 0; i < KC * PT_ROWS / WG_THREADS; ++i) {
