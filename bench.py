@@ -15,7 +15,7 @@ attention block, and every convolution of ResNet-50's bottleneck stages) under "
 of the headline workload on the host cores.
 
 `--only NAME` runs one workload alone (headline, cfg1, cfg2, cfg3-m11, cfg4, cfg4-m11,
-cfg5, resnet50) without micro-kernels or CPU baseline: the form the profiler runs.
+cfg5, resnet50, short-k) without micro-kernels or CPU baseline: the form the profiler runs.
 """
 import argparse
 import ctypes as C
@@ -358,6 +358,38 @@ def run_cfg5(roof):
     return out
 
 
+def run_short_reductions(roof):
+    """Where short reductions lose their time.  Dense products [M, K] . [K, 256] with K = 64, 128, 256 at
+    M = 50 176, 100 352, 200 704 (3136 to 12 544 tiles of 64 x 64 outputs on 1536 workgroup slots), each
+    timed as a whole call (pre-pass + main kernel) from a captured graph: a straight line through the
+    three times gives the cost of one more tile -- the marginal rate -- and what a call costs before its
+    first product (pre-pass launch, ramp-up of the first round of workgroups, drain of the last)."""
+    import torch
+    from approxtrain_amd import functors
+    lut = make_lut("MBM", 7)
+    out = {}
+    for K in (64, 128, 256):
+        B = torch.randn((K, 256), device="cuda")
+        pts = []
+        for mult in (4, 8, 16):
+            M = 12544 * mult
+            A = torch.randn((M, K), device="cuda")
+            us = device_ms_graph(lambda: functors.gemm(lut, A, B), calls=10, replays=5) * 1e3
+            pts.append((M * 256 * K, us))
+            del A
+        n = len(pts)
+        sx, sy = sum(p[0] for p in pts), sum(p[1] for p in pts)
+        sxx, sxy = sum(p[0] * p[0] for p in pts), sum(p[0] * p[1] for p in pts)
+        slope = (n * sxy - sx * sy) / (n * sxx - sx * sx)  # us per MAC
+        fixed = (sy - slope * sx) / n
+        e = {"call_us_at_3136_6272_12544_tiles": [round(p[1], 1) for p in pts],
+             "fixed_us_per_call": round(fixed, 1), "marginal_gmacs": round(1e-3 / slope, 1)}
+        if roof:
+            e["marginal_roof_frac"] = round(1e-3 / slope / roof, 4)
+        out["K=%d" % K] = e
+    return out
+
+
 RESNET50_SIZES = (("feature_maps_56_to_7", 56, 64), ("feature_maps_32_to_4_cifar", 32, 3))
 
 
@@ -377,7 +409,7 @@ def resnet50_layers(hw0, cin0):
     return layers
 
 
-def run_resnet50(roof):
+def run_resnet50(roof, only_layer=None):
     """Every convolution of ResNet-50's bottleneck stages 2-5 (the layout profile/resnet50.py:295-313
     builds: per stage one block with a strided 1x1 and a 1x1 shortcut, then identity blocks of
     1x1 -> 3x3 -> 1x1) at batch 32, MBM_7: forward, grad-input and grad-filter of each distinct layer
@@ -391,7 +423,9 @@ def run_resnet50(roof):
     gen.manual_seed(20)
     out = {}
     for label, hw0, cin0 in RESNET50_SIZES:
-        layers = resnet50_layers(hw0, cin0)
+        layers = [l for l in resnet50_layers(hw0, cin0) if only_layer is None or l[0] == only_layer]
+        if not layers:
+            continue
         total_ms = total_macs = 0.0
         per_layer = {}
         for name, hw, cin, cout, k, stride, count in layers:
@@ -432,7 +466,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="headline workload only")
-    ap.add_argument("--only", default=None, help="run one workload alone: headline, cfg1, cfg2, cfg3-m11, cfg4, cfg4-m11, cfg5, resnet50")
+    ap.add_argument("--layer", default=None, help="with --only resnet50: one layer by name, e.g. s3a_1x1/2_256_128 (both sizes)")
+    ap.add_argument("--only", default=None, help="run one workload alone: headline, cfg1, cfg2, cfg3-m11, cfg4, cfg4-m11, cfg5, resnet50, short-k")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -450,9 +485,9 @@ def main():
 
     if args.only and args.only != "headline":
         runners = {"cfg1": lambda: run_cfg1(None), "cfg2": lambda: run_cfg2(None), "cfg4": lambda: run_cfg4(None, None),
-                   "cfg3-m11": lambda: run_cfg3_wide(None, None, None),
+                   "cfg3-m11": lambda: run_cfg3_wide(None, None, None), "short-k": lambda: run_short_reductions(None),
                    "cfg4-m11": lambda: run_cfg4(None, None, tables={("MBM", 11), ("MIT", 11)}), "cfg5": lambda: run_cfg5(None),
-                   "resnet50": lambda: run_resnet50(None)}
+                   "resnet50": lambda: run_resnet50(None, args.layer)}
         if args.only not in runners:
             sys.exit("unknown workload " + args.only)
         calibration_copy(lib)
@@ -572,6 +607,7 @@ def main():
             "cfg1": run_cfg1(peak), "cfg2": run_cfg2(peak), "cfg3_MBM_11": run_cfg3_wide(peak, wide_peak, wide_pull),
             "cfg4": run_cfg4(peak, wide_peak, pull=wide_pull), "cfg5": run_cfg5(peak),
             "resnet50_convolutions_batch32": run_resnet50(peak),
+            "short_reductions_fixed_cost_and_marginal_rate": run_short_reductions(peak),
         }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(x, w, dy)
