@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace amsim {
 
@@ -97,6 +98,56 @@ __device__ __forceinline__ uint64_t add_u64_vs(uint64_t v, uint64_t s_uniform)
     uint64_t d;
     asm("v_lshl_add_u64 %0, %1, 0, %2" : "=v"(d) : "v"(v), "s"(s_uniform));
     return d;
+}
+
+// LDS byte address of a pointer into a __shared__ object
+__device__ __forceinline__ uint32_t lds_address(const void *p)
+{
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+// Byte gather from LDS into the upper half of a register: the byte arrives already shifted left by
+// 16, where the product factor wants it.  The lower half of d must be zero before (a device either
+// keeps or clears the half that such a load does not write; either way it is zero afterwards).  The
+// compiler does not know that this is a load: whoever reads the result first waits for it
+// (wait_add_u64_vs).  Issued in program order (volatile).
+__device__ __forceinline__ void lds_gather_u8_hi(uint32_t &d, uint32_t lds_byte_address)
+{
+    asm volatile("ds_read_u8_d16_hi %0, %1" : "+v"(d) : "v"(lds_byte_address));
+}
+
+// add_u64_vs after waiting until at most OUTSTANDING of the LDS / scalar-memory operations issued so
+// far are still in flight (LDS operations complete in order, so this names the gathers that have
+// landed; operations the compiler adds on its own only make the wait stricter).  Kept in program
+// order relative to the gathers (volatile): the count is only meaningful after all of them.
+template <int OUTSTANDING>
+__device__ __forceinline__ uint64_t wait_add_u64_vs(uint64_t v, uint64_t s_uniform)
+{
+    uint64_t d;
+    asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_lshl_add_u64 %0, %1, 0, %2" : "=v"(d) : "v"(v), "s"(s_uniform), "n"(OUTSTANDING));
+    return d;
+}
+
+// The same sum and a fused multiply-add, kept where they are written relative to the gathers and
+// waits above (volatile): the inner loop's instruction order is chosen by hand.
+__device__ __forceinline__ uint64_t add_u64_vs_ordered(uint64_t v, uint64_t s_uniform)
+{
+    uint64_t d;
+    asm volatile("v_lshl_add_u64 %0, %1, 0, %2" : "=v"(d) : "v"(v), "s"(s_uniform));
+    return d;
+}
+__device__ __forceinline__ void fmac_ordered(float &acc, float a, float b)
+{
+    asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc) : "v"(a), "v"(b));
+}
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
 }
 
 // Full-domain product.  `entry16` is the LUT byte (carry << 7 | mantissa

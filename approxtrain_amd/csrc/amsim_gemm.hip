@@ -68,6 +68,7 @@ struct KArgs {
     int64_t so_r, so_j, out_batch_stride;
     int batch;
     int vec_store;           // outputs of a row are contiguous (so_j == 1) and every row starts 16-byte aligned
+    int d16_keeps;           // this device's 16-bit LDS loads keep the register half they do not write (Lut::d16_keeps)
     Epilogue ep;
     // A launch covers up to two row segments, workgroups of seg[0] first in dispatch order:
     // seg[0] the split-reduction tail (if any), seg[1] the main part.
@@ -201,6 +202,12 @@ __device__ __forceinline__ void fill_rowinfo(const PDesc &p, int64_t R, int64_t 
 // LUTG   false: byte LUT image resident in LDS (mantissa width <= 7)
 //        true:  16-bit LUT image gathered from global memory through L2 / MALL
 //               (widths 8..11; a 2^22-entry table does not fit the 160 KB LDS)
+#ifndef AMSIM_D16
+#define AMSIM_D16 1
+#endif
+#ifndef AMSIM_D16_PU
+#define AMSIM_D16_PU 4
+#endif
 constexpr int WR_KSLICES = 0;  // value of WR that selects the reduction-slice arrangement
 
 template <int TN, int WR, int PK, int STAGE, bool LUTG>
@@ -215,6 +222,7 @@ void lutgemm_kernel(KArgs a)
     constexpr int GS = ROWS + 1;  // padded group stride (in uint4): conflict-free transposing stores
     constexpr int ELEMS = ROWS * KC / WG_THREADS;
     constexpr int QUADS = ELEMS / 4;
+    constexpr bool D16_LOOP = AMSIM_D16 && !LUTG && TN % 2 == 0;  // the hand-ordered inner loop (below)
 
     __shared__ __align__(16) uint8_t lut_s[LUTG ? (KSLICES ? 3 * TN * 64 * sizeof(float) : 16) : LUT_LDS_BYTES];
     const uint16_t *__restrict__ lut_g = reinterpret_cast<const uint16_t *>(a.lut_img);
@@ -541,6 +549,7 @@ void lutgemm_kernel(KArgs a)
     if (!LUTG) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const int lrow = wr * 64 + lane;
     const int mshift = 23 - m;
+    const uint32_t lut_base = lds_address(lut_s);
 
     // Touching the next chunk's pre-decoded uniform operand (one lane per 128-byte line of this
     // wavefront's 2 KB) a chunk ahead brings it into L2 when it streams from HBM (filter gradients,
@@ -594,6 +603,79 @@ void lutgemm_kernel(KArgs a)
             fast = spans_compatible(span_word(wave_union(mine)), q_span);
         }
         if (fast) {
+          if constexpr (D16_LOOP) {
+            // Gathers that deliver the byte already shifted (upper register half): the factors of two
+            // columns are then one 64-bit add as well -- per pair of products two instructions that read
+            // scalar registers instead of three.  Written out as a software pipeline over "units" of PU
+            // column pairs: while one unit's factors and multiply-adds issue, the next unit's addresses and
+            // gathers go out between them, so that an instruction that reads scalar registers is always
+            // followed by one that does not.  (The uniform operand's words of a group of four rows are
+            // loaded and waited for together: scalar loads return out of order, so waiting for one drains
+            // the gathers in flight as well -- loading half a group ahead doubled those drains and lost 3 %.)
+            constexpr int TN2 = (TN + 1) / 2;
+            constexpr int PU = AMSIM_D16_PU < TN2 ? AMSIM_D16_PU : TN2;  // column pairs per unit
+            constexpr int UPR = TN2 / PU;                               // units per reduction row
+            constexpr int NU = KG * UPR;                                // units of a group of rows
+            cq1_t qrow = qw + qoff + g_first * (KG * QT);
+            // The gathers' destinations: a gather writes the upper half of its register; the lower half
+            // must read as zero.  Devices differ in what such a load does to the other half (kept, or
+            // cleared -- probed once per device): where it is kept, the registers start each chunk as zero.
+            uint32_t Lh[2][2 * PU];
+            if (a.d16_keeps) {
+#pragma unroll
+                for (int i = 0; i < 4 * PU; ++i) asm volatile("v_mov_b32 %0, 0" : "=v"(Lh[i / (2 * PU)][i % (2 * PU)]));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4 * PU; ++i) asm volatile("" : "=v"(Lh[i / (2 * PU)][i % (2 * PU)]));
+            }
+#pragma unroll 1
+            for (int g = g_first; g < g_last; ++g) {
+                uint64_t qw2[KG][TN2];
+#pragma unroll
+                for (int r = 0; r < KG; ++r)
+#pragma unroll
+                    for (int j = 0; j < TN2; ++j) qw2[r][j] = reinterpret_cast<cq2_t>(qrow + r * QT)[j];
+                const uint4 p4 = Pt4[g * GS + lrow];
+                const uint32_t praw[KG] = {p4.x, p4.y, p4.z, p4.w};
+                float ta[KG];
+                uint64_t iab2[KG];
+#pragma unroll
+                for (int r = 0; r < KG; ++r) {
+                    ta[r] = u2f(praw[r] & 0xff800000u);
+                    const uint32_t iab = __builtin_amdgcn_ubfe(praw[r], (uint32_t)mshift, (uint32_t)m) + lut_base;
+                    iab2[r] = ((uint64_t)iab << 32) | iab;
+                }
+                qrow += KG * QT;
+                auto issue = [&](auto uc, auto ic) {
+                    constexpr int u = decltype(uc)::value, i = decltype(ic)::value;
+                    constexpr int r = u / UPR, pr = (u % UPR) * PU + i;
+                    const uint64_t qi2 = qw2[r][pr] & 0x007fffff007fffffull;
+                    const uint64_t li2 = add_u64_vs_ordered(iab2[r], qi2);
+                    lds_gather_u8_hi(Lh[u & 1][2 * i], (uint32_t)li2);
+                    lds_gather_u8_hi(Lh[u & 1][2 * i + 1], (uint32_t)(li2 >> 32));
+                };
+                static_for<0, PU>([&](auto ic) { issue(std::integral_constant<int, 0>{}, ic); });
+                static_for<0, NU>([&](auto uc) {
+                    constexpr int u = decltype(uc)::value;
+                    constexpr int r = u / UPR;
+                    // (a fence per unit: left alone the scheduler hoists every mask operation of the group to
+                    // the loop's top and spills their results)
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<0, PU>([&](auto ic) {
+                        constexpr int i = decltype(ic)::value;
+                        constexpr int pr = (u % UPR) * PU + i;
+                        // gathers issued after this pair's: the rest of this unit and what the next unit
+                        // has sent so far
+                        constexpr int younger = u + 1 < NU ? 2 * (PU - 1) : 2 * (PU - 1 - i);
+                        const uint64_t qt2 = qw2[r][pr] & 0xff800000ff800000ull;
+                        const uint64_t g2 = wait_add_u64_vs<younger>(((uint64_t)Lh[u & 1][2 * i + 1] << 32) | Lh[u & 1][2 * i], qt2);
+                        fmac_ordered(acc[2 * pr], ta[r], u2f((uint32_t)g2));
+                        if constexpr (u + 1 < NU) issue(std::integral_constant<int, u + 1>{}, ic);
+                        fmac_ordered(acc[2 * pr + 1], ta[r], u2f((uint32_t)(g2 >> 32)));
+                    });
+                });
+            }
+          } else {
             cq1_t qrow = qw + qoff + g_first * (KG * QT);
 #pragma unroll 1
             for (int g = g_first; g < g_last; ++g) {
@@ -640,6 +722,7 @@ void lutgemm_kernel(KArgs a)
                 }
                 qrow += KG * QT;
             }
+          }
         } else {
             // rare: the uniform operand's raw bits come from where it lies, not from the workspace
             const uint32_t *Pt = reinterpret_cast<const uint32_t *>(Pt4);
@@ -1238,6 +1321,7 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
     ka.batch = d.batch;
     ka.ep = Epilogue{d.bias_j, d.bias_r, d.act, d.omap};
     ka.vec_store = (d.so_j == 1 && d.so_r % 4 == 0 && d.out_batch_stride % 4 == 0 && aligned16(d.out)) ? 1 : 0;
+    ka.d16_keeps = lut.d16_keeps;
 
     const int rows = pl.WR > 1 ? 64 * pl.WR : 64, wc = pl.WR == WR_KSLICES ? 1 : 4 / pl.WR;
     const int64_t jchunks = (d.J + pl.TN - 1) / pl.TN;
@@ -1279,6 +1363,43 @@ int run_gemm(const Lut &lut, const GemmDesc &d, void *workspace, size_t workspac
         launch_reduce(ra, stream);
         AMSIM_HIP_CHECK(hipGetLastError());
     }
+    return AMSIM_OK;
+}
+
+// What does a 16-bit LDS load do to the register half it does not write?  One wavefront loads a
+// byte into the upper half of a register that holds all ones.
+__global__ __launch_bounds__(64) void d16_probe_kernel(uint32_t *out)
+{
+    __shared__ uint32_t cell[64];
+    cell[threadIdx.x] = 0x5au;
+    __syncthreads();
+    uint32_t d = 0xffffffffu;
+    asm volatile("ds_read_u8_d16_hi %0, %1\n\ts_waitcnt lgkmcnt(0)" : "+v"(d) : "v"(lds_address(&cell[threadIdx.x])));
+    out[threadIdx.x] = d;
+}
+
+int probe_lds_d16_keeps(int *keeps)
+{
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<int> cache[MAX_DEVICES];  // 0 unknown, 1 clears, 2 keeps
+    int dev = 0;
+    AMSIM_HIP_CHECK(hipGetDevice(&dev));
+    if (dev >= 0 && dev < MAX_DEVICES && cache[dev].load() != 0) {
+        *keeps = cache[dev].load() == 2;
+        return AMSIM_OK;
+    }
+    uint32_t *d_out = nullptr, h_out[64];
+    AMSIM_HIP_CHECK(hipMalloc(reinterpret_cast<void **>(&d_out), sizeof(h_out)));
+    d16_probe_kernel<<<1, 64, 0, nullptr>>>(d_out);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpy(h_out, d_out, sizeof(h_out), hipMemcpyDeviceToHost);
+    (void)hipFree(d_out);
+    if (e != hipSuccess) return fail(AMSIM_ERR_HIP, std::string("LDS load probe: ") + hipGetErrorString(e));
+    for (int i = 0; i < 64; ++i)
+        if (h_out[i] != h_out[0] || (h_out[0] != 0x005a0000u && h_out[0] != 0x005affffu))
+            return fail(AMSIM_ERR_UNSUPPORTED, "unexpected result of a 16-bit LDS load on this device");
+    *keeps = h_out[0] == 0x005affffu;
+    if (dev >= 0 && dev < MAX_DEVICES) cache[dev].store(*keeps ? 2 : 1);
     return AMSIM_OK;
 }
 

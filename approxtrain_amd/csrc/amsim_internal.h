@@ -41,6 +41,8 @@ struct Lut {
     // m > 7 only: carry << 15 | mantissa << (15 - m), and its transpose
     uint16_t *img16_ab = nullptr;
     uint16_t *img16_ba = nullptr;
+    // this device's 16-bit LDS loads keep (1) or clear (0) the register half they do not write
+    int d16_keeps = 0;
 };
 
 }  // namespace amsim
@@ -115,6 +117,8 @@ struct GemmDesc {
 int device_compute_units();
 // AMSIM_OK when the handle's images live on the current device, else AMSIM_ERR_INVALID.
 int check_lut_device(const Lut &lut);
+// how 16-bit LDS loads treat the other register half on the current device (probed once per device)
+int probe_lds_d16_keeps(int *keeps);
 
 size_t gemm_workspace_bytes(int64_t R, int64_t J, int64_t K, int batch, int q_batches);
 void gemm_plan_info(int64_t R, int64_t J, int64_t K, int batch, int q_batches, bool split_k, int waves64, int64_t info[8]);

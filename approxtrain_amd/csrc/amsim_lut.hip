@@ -103,6 +103,10 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
         if ((rc = upload(&l.img16_ab, ab)) != AMSIM_OK) return rc;
         if ((rc = upload(&l.img16_ba, ba)) != AMSIM_OK) return rc;
     }
+    if ((rc = probe_lds_d16_keeps(&l.d16_keeps)) != AMSIM_OK) {
+        lut_free(l);
+        return rc;
+    }
     *out = l;
     return AMSIM_OK;
 }
