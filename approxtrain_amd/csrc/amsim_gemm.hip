@@ -19,10 +19,12 @@
 //     gathers computed on the fly: no im2col / flipped-filter temporaries in
 //     HBM -- in a [k/4][r][4] layout that a lane reads back 16 bytes at a time.
 //   * per pair of MACs: one v_lshl_add_u64 (two LUT addresses: the lane's
-//     mantissa index in both halves + a pair of row offsets), two ds_read_u8,
-//     two v_lshl_add_u32 (LUT byte shifted into the mantissa/carry position
-//     PLUS the uniform operand's sign|exponent bits = q_pow2 * 1.mant * 2^carry
-//     as a float), two v_fma with the lane operand's power of two (accumulate).  The product inside the fma is
+//     mantissa index in both halves + a pair of row offsets), two
+//     ds_read_u8_d16_hi (the LUT byte lands in the upper register half, i.e.
+//     shifted into the mantissa/carry position), one v_lshl_add_u64 (the two
+//     gathered registers PLUS the uniform operand's sign|exponent bits of both
+//     columns = q_pow2 * 1.mant * 2^carry as two floats), two v_fma with the
+//     lane operand's power of two (accumulate).  The product inside the fma is
 //     exact (power of two times an 8-bit significand), so the fused
 //     multiply-add rounds exactly like the reference's product-then-add.
 //     Zero uniform operands select an all-zero LUT row, zero lane operands a

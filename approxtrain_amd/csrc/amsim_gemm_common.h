@@ -17,7 +17,7 @@ constexpr int WG_THREADS = 256;
 constexpr int LUT_LDS_BYTES = 16384 + 128;   // 2^(2m) entries + one all-zero row of 2^m entries (m <= 7)
 constexpr int WAVES_PER_SIMD = 6;             // occupancy the 64-row kernels are compiled for
 constexpr int NUM_XCD = 8;                    // accelerator dies, each with a private L2
-constexpr double MACS_PER_CU_S = 13.0e12 / 256;  // planner's price of a MAC: what one compute unit sustains
+constexpr double MACS_PER_CU_S = 15.0e12 / 256;  // planner's price of a MAC: what one compute unit sustains
 constexpr double PARTIAL_BYTES_PER_S = 3.0e12;   // planner's price of writing + re-reading partial sums
 constexpr double WORKGROUP_START_S = 3.5e-6;     // planner's price of a round of workgroup starts (LUT staging, first loads)
 

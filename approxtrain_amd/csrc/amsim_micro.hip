@@ -20,6 +20,9 @@ constexpr int MICRO_UNROLL = 16;
 //          addresses), two v_lshl_add_u32 (VGPR << 16 + SGPR), two v_fma_f32 -- 5 ops per two slots
 //       6: the row-staged GEMM's pair per product: v_mad_u32_u16 (16-bit half * 256 + SGPR) feeding a
 //          v_fma_f32 two instructions later -- 2 ops per slot
+//       7: the GEMM's mix per pair of MACs when the gathers deliver the byte already shifted: two
+//          v_lshl_add_u64 (VGPR pair + SGPR pair: two LUT addresses, two product factors), two
+//          v_fma_f32, alternating -- 2 ops per slot
 template <int VMODE>
 __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, float *sink, long long *clk)
 {
@@ -47,6 +50,13 @@ __global__ __launch_bounds__(MICRO_THREADS) void micro_valu_kernel(int iters, fl
                 asm volatile("v_lshl_add_u32 %0, %1, 16, %2" : "=v"(t1) : "v"((uint32_t)(t2 >> 32)), "s"(iters));
                 asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j]) : "v"(c2), "v"(t0));
                 asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j + 1]) : "v"(c2), "v"(t1));
+            } else if (VMODE == 7) {
+                if (j & 1) continue;
+                uint64_t t2, u2;
+                asm volatile("v_lshl_add_u64 %0, %1, 0, %2" : "=v"(t2) : "v"(pair), "s"(spair));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j]) : "v"(c2), "v"((uint32_t)t2));
+                asm volatile("v_lshl_add_u64 %0, %1, 0, %2" : "=v"(u2) : "v"(t2), "s"(spair));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(a[j + 1]) : "v"(c2), "v"((uint32_t)(u2 >> 32)));
             } else if (VMODE == 6) {
                 if (j & 1) continue;
                 uint32_t t0, t1;
@@ -323,7 +333,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
                      double *ops_per_launch)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (kind < 0 || (kind > 6 && kind < 10) || (kind > 16 && kind < 21) || kind > 22 || blocks < 1 || iters < 1 || reps < 1 || !sink || !ms_per_launch || !ops_per_launch)
+    if (kind < 0 || (kind > 6 && kind < 10) || (kind > 17 && kind < 21) || kind > 22 || blocks < 1 || iters < 1 || reps < 1 || !sink || !ms_per_launch || !ops_per_launch)
         return fail(AMSIM_ERR_INVALID, "bad microbench arguments");
     hipEvent_t e0, e1;
     AMSIM_HIP_CHECK(hipEventCreate(&e0));
@@ -338,6 +348,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
         case 14: micro_valu_kernel<4><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 15: micro_valu_kernel<5><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 16: micro_valu_kernel<6><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
+        case 17: micro_valu_kernel<7><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink, (long long *)(sink + 512)); break;
         case 21: micro_lds_fit_kernel<0><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
         case 22: micro_lds_fit_kernel<1><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
         case 1: micro_lds_kernel<0><<<blocks, MICRO_THREADS, 0, stream>>>(iters, sink); break;
@@ -359,7 +370,7 @@ int amsim_microbench(int kind, int blocks, int iters, int reps, void *stream_, f
     AMSIM_HIP_CHECK(hipEventDestroy(e1));
     AMSIM_HIP_CHECK(hipGetLastError());
     *ms_per_launch = (double)ms / reps;
-    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4.0 : kind == 15 ? 2.5 : kind == 16 ? 2.0 : 1.0);
+    *ops_per_launch = (double)blocks * MICRO_THREADS * (double)iters * MICRO_UNROLL * (kind == 14 ? 4.0 : kind == 15 ? 2.5 : (kind == 16 || kind == 17) ? 2.0 : 1.0);
     return AMSIM_OK;
 }
 

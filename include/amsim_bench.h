@@ -22,12 +22,13 @@ extern "C" {
 int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t info[8]);
 /* Micro-kernels that measure, on the current device, the VALU issue rate
  * (kind 0 / 10: independent FP32 FMAs; 11..13: v_add_u32, v_lshl_add_u32,
- * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's mix, 5 instructions per two MACs;
- * 16: the row-staged GEMM's pair per product, a 16-bit multiply-add that forms the factor + an FMA) and
+ * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's earlier mix, 5 instructions per two MACs;
+ * 16: the row-staged GEMM's pair per product, a 16-bit multiply-add that forms the factor + an FMA;
+ * 17: the GEMM inner loop's mix, 4 instructions per two MACs: two 64-bit adds of a scalar pair, two FMAs) and
  * the LDS gather rate (kinds 1..6: u8 / u16 / b32 reads, lanes inside one
  * 128-element row or scattered, with 64 KB of LDS per workgroup; kinds 21 / 22: the u8 pair
  * again at the GEMM kernel's own LDS footprint and occupancy, reads software-pipelined).
- * Kinds 10..16 also leave two 64-bit counts at sink[512..515]: the shader-clock ticks of one
+ * Kinds 10..17 also leave two 64-bit counts at sink[512..515]: the shader-clock ticks of one
  * workgroup's loop and the same interval in 100 MHz ticks (their ratio is the clock).  Launches
  * `reps` times on `stream`, timed with HIP events; `sink` is any device buffer
  * of >= 256 floats. */
