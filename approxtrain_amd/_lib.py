@@ -41,6 +41,7 @@ SIGNATURES = {
     "amsim_gemm_workspace_bytes": (_sz, [_i, _i, _i64, _i64, _i64, _i64]),
     "amsim_gemm_workspace_bytes_for": (_sz, [_p, _i, _i, _i64, _i64, _i64, _i64]),
     "amsim_gemm_plan_info": (_i, [_i, _i, _i64, _i64, _i64, _i64, C.POINTER(_i64)]),
+    "amsim_lut_force_gather_zeroing": (_i, [_p, _i, C.POINTER(_i)]),
     "amsim_gemm_f32": (_i, [_p, _i, _i, _i, _i64, _i64, _i64, _f, _i64, _f, _i64, _f, _i64,
                             _i64, _i64, _i64, _i64, _p, _sz, _p]),
     "amsim_convam_workspace_bytes": (_sz, [_i] * 7),

@@ -43,6 +43,7 @@ struct Lut {
     uint16_t *img16_ba = nullptr;
     // this device's 16-bit LDS loads keep (1) or clear (0) the register half they do not write
     int d16_keeps = 0;
+    int d16_keeps_probed = 0;  // the probe's answer (d16_keeps may be forced to 1 by a test hook)
 };
 
 }  // namespace amsim

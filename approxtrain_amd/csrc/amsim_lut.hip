@@ -2,6 +2,7 @@
 // the device images the kernels read (the counterpart of the cudaMalloc +
 // texture object of cuda/approx_mul_lut.cu:24-48).
 #include "amsim_internal.h"
+#include "amsim_bench.h"
 
 #include <atomic>
 #include <cstdio>
@@ -107,6 +108,7 @@ static int build_images(int m, const std::vector<uint8_t> &carry, const std::vec
         lut_free(l);
         return rc;
     }
+    l.d16_keeps_probed = l.d16_keeps;
     *out = l;
     return AMSIM_OK;
 }
@@ -260,6 +262,15 @@ int amsim_lut_set_split_k(amsim_lut_t lut, int mode)
     if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
     if (mode < -1 || mode > 1) return fail(AMSIM_ERR_INVALID, "split mode must be -1 (process default), 0 or 1");
     lut->l.split_k = mode;
+    return AMSIM_OK;
+}
+
+int amsim_lut_force_gather_zeroing(amsim_lut_t lut, int on, int *probed)
+{
+    if (lut == nullptr) return fail(AMSIM_ERR_INVALID, "null LUT handle");
+    if (on != 0 && on != 1) return fail(AMSIM_ERR_INVALID, "on must be 0 or 1");
+    lut->l.d16_keeps = on ? 1 : lut->l.d16_keeps_probed;
+    if (probed) *probed = lut->l.d16_keeps_probed;
     return AMSIM_OK;
 }
 

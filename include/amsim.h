@@ -68,7 +68,11 @@ int amsim_device_info(char *arch, size_t arch_len, int *compute_units);
  * file format for.
  * amsim_lut_create takes the entries from host memory; entry_bytes is 1
  * (layout above, m <= 7) or 4 (legacy layout of lut/AMsimulator.inl:18-20:
- * bit 31 = carry, bits 22..0 = mantissa in place; m <= 11). */
+ * bit 31 = carry, bits 22..0 = mantissa in place; m <= 11).
+ * Both upload the table images to the current device and wait for the copies; the first handle
+ * created on a device also runs a one-wavefront probe kernel there (how 16-bit LDS loads treat
+ * the other register half, which the GEMM kernels adapt to).  Create handles outside stream
+ * capture. */
 int amsim_lut_load_file(const char *path, amsim_lut_t *out);
 int amsim_lut_create(const void *entries, size_t n_bytes, int mant_width, int entry_bytes, amsim_lut_t *out);
 int amsim_lut_destroy(amsim_lut_t lut);

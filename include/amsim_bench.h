@@ -20,6 +20,13 @@ extern "C" {
  * reduction, chunks (of 32) per split, rows in the main part, splits of the tail rows' reduction
  * (0 = no tail), chunks per tail split, chunks in all}.  For tests and tuning. */
 int amsim_gemm_plan_info(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t info[8]);
+/* Test hook.  The LDS-table GEMM gathers table bytes into the upper half of a register whose lower
+ * half must read as zero; whether a 16-bit LDS load keeps or clears the half it does not write
+ * differs between devices and is probed once per device when a handle is created.  Where it is
+ * kept, the kernel zeroes those registers once per reduction chunk.  on = 1 makes calls through
+ * this handle take that branch whatever the probe said (results must not change), on = 0 restores
+ * the probe's answer; *probed (may be NULL) receives the probe's answer: 1 = kept, 0 = cleared. */
+int amsim_lut_force_gather_zeroing(amsim_lut_t lut, int on, int *probed);
 /* Micro-kernels that measure, on the current device, the VALU issue rate
  * (kind 0 / 10: independent FP32 FMAs; 11..13: v_add_u32, v_lshl_add_u32,
  * v_mul_f32; 14: a 4-op mix; 15: the GEMM inner loop's earlier mix, 5 instructions per two MACs;

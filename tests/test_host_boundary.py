@@ -23,7 +23,8 @@ def declared_symbols(header="amsim.h"):
     return sorted(set(re.findall(r"\b(amsim_[a-z0-9_]+)\s*\(", text)))
 
 
-BENCH_ONLY = {"amsim_microbench", "amsim_microbench_wide", "amsim_calibration_copy", "amsim_gemm_plan_info"}
+BENCH_ONLY = {"amsim_microbench", "amsim_microbench_wide", "amsim_calibration_copy", "amsim_gemm_plan_info",
+              "amsim_lut_force_gather_zeroing"}
 
 
 def test_library_loads_and_exports_every_declared_symbol():
